@@ -802,7 +802,7 @@ DEV void lean_body(const LeanArgs& args, const int by, const LeanDyn* const dyn 
                 // decode of the current one (round 4 requested a whole load, waited for all of it, decoded it: one exposed round trip
                 // per pass).  EVERY request is unconditional -- indices past the end are clamped to the last item, a line that is in
                 // flight anyway -- in the first load's straight-line code and in the loop body alike, same order: the compiler's
-                // count of the requests in flight is exact on both edges into the loop (tests/test_lean_isa.py).
+                // count of the requests in flight is exact on both edges into the loop.
                 const u32* const lastp = wptr + (size_t)(n - 1) * STEP;
                 // (a request past the end is lane 0's words of the last item for every lane: one 16-byte line, not another 64 x 4 BITS bytes)
                 auto request = [&](LaneWords<BITS>& w, int q) { load_lane_words<BITS>(q < n ? wptr + (size_t)q * STEP : lastp, q < n ? lane : 0, w); };
