@@ -104,6 +104,14 @@ PROTOTYPES = {
     "exl2_chain_overlap_end": (ci, [C.POINTER(ci)]),
     "exl2_chain_route_counts": (ci, [C.POINTER(C.c_longlong), C.POINTER(C.c_longlong), ci]),
     "exl2_prefill_route_info": (ci, [C.POINTER(ci)]),
+    # unquantized models (csrc/dense.hip, rowops.hip, latent_attn.hip)
+    "exl2_dense_linear": (ci, [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, cll, cll, cll, cll, vp, ci, vp, vp, vp, ci, ci, cf, vp]),
+    "exl2_embed_scale": (ci, [vp, vp, vp, vp, ci, ci, ci, ci, cf, vp]),
+    "exl2_rms_rows": (ci, [vp, ci, vp, ci, vp, ci, ci, vp, ci, ci, ci, cf, vp]),
+    "exl2_post_norm": (ci, [vp, vp, vp, vp, ci, ci, ci, cf, cf, vp, vp, vp, ci, ci, vp]),
+    "exl2_moe_route_scored": (ci, [vp, vp, vp, vp, ci, ci, ci, cf, ci, vp, vp, vp, vp]),
+    "exl2_latent_append": (ci, [vp, ci, vp, cf, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, ci, vp, vp]),
+    "exl2_latent_attn": (ci, [vp, ci, ci, ci, vp, vp, ci, vp, vp, vp, ci, vp, ci, ci, ci, ci, ci, ci, vp, cf, ci, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

@@ -34,7 +34,10 @@ def build(force: bool = False, verbose: bool = False) -> str:
         return OUT
     from concurrent.futures import ThreadPoolExecutor
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    flags = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-unused-value", "-I", CSRC]
+    # (no packed-fp32 instructions: the compiler forms them from ordinary float code by itself and some forms have misbehaved on
+    # this hardware generation)
+    flags = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-unused-value", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-I", CSRC]
     headers = glob.glob(os.path.join(CSRC, "*.h"))
     hdr_time = max(os.path.getmtime(f) for f in headers) if headers else 0.0
     objs, jobs = [], []

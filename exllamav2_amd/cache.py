@@ -102,3 +102,75 @@ class ExLlamaV2Cache_Q4(ExLlamaV2Cache):
     def footprint(self) -> int:
         ts = self.key_states + self.value_states + self.key_scales + self.value_scales
         return sum(t.numel() * t.element_size() for t in ts)
+
+
+class PagePool:
+    """Host-side allocator of cache pages and sequence slots for paged caches that several requests share.
+
+    A sequence holds one slot (a row of the block table) and as many pages as its tokens need; both go back to the free lists when
+    the sequence ends and are handed out again (most recently freed first).  The block table lives on the host and is mirrored to
+    the device once per step (`device_table`), so kernels reach a token's row as
+    `pages[block_table[slot, pos // page_size], pos % page_size]`."""
+
+    def __init__(self, num_pages: int, page_size: int = PAGE_SIZE, max_seqs: int = 4, device="cuda:0"):
+        if num_pages <= 0 or page_size <= 0 or max_seqs <= 0:
+            raise ValueError("PagePool: sizes must be positive")
+        self.num_pages, self.page_size, self.max_seqs = num_pages, page_size, max_seqs
+        self.device = torch.device(device)
+        self.free_pages = list(range(num_pages - 1, -1, -1))
+        self.free_slots = list(range(max_seqs - 1, -1, -1))
+        self.table = torch.zeros((max_seqs, num_pages), dtype=torch.int32)
+        self.seq_pages = {}                                   # slot -> number of pages it holds
+        self.seq_len = {}                                     # slot -> tokens cached
+        self._dev_table = torch.zeros((max_seqs, num_pages), dtype=torch.int32, device=self.device)
+        self._dirty = True
+
+    def open(self) -> int:
+        if not self.free_slots:
+            raise RuntimeError(f"PagePool: all {self.max_seqs} sequence slots are in use")
+        slot = self.free_slots.pop()
+        self.seq_pages[slot] = 0
+        self.seq_len[slot] = 0
+        return slot
+
+    def extend(self, slot: int, n_tokens: int) -> int:
+        """Make room for n_tokens more tokens of the sequence; returns the position of the first of them."""
+        start = self.seq_len[slot]
+        need = -(-(start + n_tokens) // self.page_size)
+        while self.seq_pages[slot] < need:
+            if not self.free_pages:
+                raise RuntimeError(f"PagePool: out of cache pages ({self.num_pages} x {self.page_size} tokens)")
+            self.table[slot, self.seq_pages[slot]] = self.free_pages.pop()
+            self.seq_pages[slot] += 1
+            self._dirty = True
+        self.seq_len[slot] = start + n_tokens
+        return start
+
+    def close(self, slot: int) -> None:
+        for i in range(self.seq_pages.pop(slot) - 1, -1, -1):
+            self.free_pages.append(int(self.table[slot, i]))
+        del self.seq_len[slot]
+        self.free_slots.append(slot)
+
+    def device_table(self) -> torch.Tensor:
+        if self._dirty:
+            self._dev_table.copy_(self.table)
+            self._dirty = False
+        return self._dev_table
+
+
+class LatentCache:
+    """Paged cache of latent attention: one pool tensor [pages, page_size, kv_rank + rot_dim] per layer that OWNS its keys and
+    values (a layer that attends over another layer's latents holds nothing: `owner[layer]` names whose rows it reads).  Rows are
+    written by exl2_latent_append and read by exl2_latent_attn through the pool's block table."""
+
+    def __init__(self, pool: PagePool, row_widths: dict, owner: dict, dtype):
+        self.pool, self.owner, self.dtype = pool, dict(owner), dtype
+        self.rows = {layer: torch.zeros((pool.num_pages, pool.page_size, width), dtype=dtype, device=pool.device)
+                     for layer, width in row_widths.items()}
+
+    def layer(self, layer_idx: int) -> torch.Tensor:
+        return self.rows[self.owner[layer_idx]]
+
+    def footprint(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.rows.values())

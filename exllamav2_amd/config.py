@@ -49,3 +49,29 @@ class ExLlamaV2Config:
                  num_key_value_heads=2, head_dim=64, vocab_size=320, max_seq_len=512, max_input_len=64)
         d.update(kw)
         return ExLlamaV2Config(**d)
+
+
+@dataclass
+class LayeredConfig:
+    """A model described layer by layer in its config.json: `layers` is a list of {"type": <mixer kind>, "mixer": {sizes},
+    "mlp": {"kind": "dense" | "moe", ...} | None}; tensors of layer i are named `l<i>.*`.  Every size and constant comes from
+    the file (or a tensor's shape); nothing is assumed equal across layers."""
+    architecture: str = ""
+    vocab: int = 0
+    width: int = 0
+    norm_eps: float = 1e-5
+    postln_alpha: float = 1.0
+    embedding_scale: float = 1.0
+    layers: list = field(default_factory=list)
+
+    @staticmethod
+    def from_dict(d: dict) -> "LayeredConfig":
+        try:
+            cfg = LayeredConfig(architecture=str(d["architecture"]), vocab=int(d["vocab"]), width=int(d["width"]),
+                                norm_eps=float(d["norm"]["eps"]), postln_alpha=float(d["postln_alpha"]),
+                                embedding_scale=float(d["embedding"]["scale"]), layers=list(d["layers"]))
+        except KeyError as e:
+            raise RuntimeError(f"config.json: missing key {e}") from e
+        if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:
+            raise RuntimeError("config.json: vocab, width and layers must be given")
+        return cfg

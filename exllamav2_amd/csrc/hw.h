@@ -140,6 +140,22 @@ DEV f32x4 mfma_16x16x32_f16(f16x8 a, f16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+
+// ---- bfloat16 (stored as its 16 bits): widening is a shift, narrowing rounds to nearest even ----------------------------
+DEV float bf16_to_f32(u16 v) { return as_f32((u32)v << 16); }
+DEV u16 f32_to_bf16(float f)
+{
+    u32 u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40u);      // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (u16)(u >> 16);
+}
+// D[16x16] += A[16x32] * B[32x16], bf16 in (8 values = 4 dwords per lane, same lane map as mfma_16x16x32_f16) / fp32 accumulate
+DEV f32x4 mfma_16x16x32_bf16(u32x4 a, u32x4 b, f32x4 c) {
+    typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
 // fp32 += dot(half2, half2): v_dot2_f32_f16
 DEV float dot2_f32_f16(f16x2 a, f16x2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
 

@@ -1,0 +1,282 @@
+// rowops.hip -- the row-wise steps around the dense linears (dense.hip), fp32 arithmetic throughout, + their C ABI:
+//   * embedding gather times a scale into the fp32 residual stream (+ its operand-dtype copy for the next linear),
+//   * RMS norm of a (strided) fp32 row slice with a plain weight w or a zero-centred one (1 + w), optional row gather,
+//   * the post-norm residual step  x <- norm(alpha x + y) (1 + w), where y is a linear's fp32 output or the weighted sum of a
+//     token's chosen experts (identity experts contribute the token's own x),
+//   * the sparse-MoE router (softmax over all experts, selection by score + correction, weights from the uncorrected scores) and
+//     the per-expert row lists the grouped linear reads.
+// Element type T of weights / operand copies: u16 = bfloat16 bits, float.
+#include "hw.h"
+#include "errors.h"
+
+template <typename T> DEV float ro_ld(const T* p);
+template <> DEV float ro_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
+template <> DEV float ro_ld<float>(const float* p) { return *p; }
+template <typename T> DEV void ro_st(T* p, float v);
+template <> DEV void ro_st<u16>(u16* p, float v) { *p = f32_to_bf16(v); }
+template <> DEV void ro_st<float>(float* p, float v) { *p = v; }
+
+// sum over the 256 threads of a workgroup (every thread gets it)
+DEV float block_sum_256(float v, float* part)
+{
+    v = wave_allreduce_add(v);
+    block_sync();
+    if (lane_id() == 0) part[wave_id()] = v;
+    block_sync();
+    return part[0] + part[1] + part[2] + part[3];
+}
+
+// ---- embedding ------------------------------------------------------------------------------------------------------------
+
+template <typename T>
+KERNEL void __launch_bounds__(256) embed_scale_kernel(const T* table, const int* ids, float* x32, T* xh, int width, int vocab, float scale)
+{
+    const int r = bid_x();
+    int id = ids[r];
+    id = min(max(id, 0), vocab - 1);
+    const T* src = table + (long long)id * width;
+    for (int i = tid(); i < width; i += 256)
+    {
+        const float v = ro_ld<T>(src + i) * scale;
+        x32[(long long)r * width + i] = v;
+        if (xh && (void*)xh != (void*)x32) ro_st<T>(xh + (long long)r * width + i, v);
+    }
+}
+
+// ---- RMS norm of a row slice ------------------------------------------------------------------------------------------------
+
+template <typename T>
+KERNEL void __launch_bounds__(256) rms_rows_kernel(const float* x, int ldx, const T* w, int one_plus, void* y, int ldy, int y_f32,
+                                                    const int* row_idx, int dim, float eps)
+{
+    SHARED float part[4];
+    const int r = bid_x();
+    const float* xr = x + (long long)(row_idx ? row_idx[r] : r) * ldx;
+    float ss = 0.0f;
+    for (int i = tid(); i < dim; i += 256) { const float v = xr[i]; ss = fmaf(v, v, ss); }
+    ss = block_sum_256(ss, part);
+    const float rinv = 1.0f / sqrtf(ss / (float)dim + eps);
+    for (int i = tid(); i < dim; i += 256)
+    {
+        const float wv = ro_ld<T>(w + i) + (one_plus ? 1.0f : 0.0f);
+        const float v = xr[i] * rinv * wv;
+        if (y_f32) ((float*)y)[(long long)r * ldy + i] = v; else ro_st<T>((T*)y + (long long)r * ldy + i, v);
+    }
+}
+
+// ---- x <- norm(alpha x + y) (1 + w) -------------------------------------------------------------------------------------------
+
+struct PostNormArgs
+{
+    float* x; void* xh; const float* y; const void* w;
+    int width; float alpha, eps;
+    // sparse-MoE form (y == nullptr): y = sum_k moe_w[r, k] * (moe_ids[r, k] >= n_real ? x[r] : moe_y[r * top + k])
+    const float* moe_y; const int* moe_ids; const float* moe_w; int top, n_real;
+};
+
+template <typename T>
+KERNEL void __launch_bounds__(256) post_norm_kernel(const PostNormArgs a)
+{
+    DYN_SMEM(smem);
+    SHARED float part[4];
+    float* v = (float*)smem;                                     // the row before the norm
+    const int r = bid_x();
+    float* xr = a.x + (long long)r * a.width;
+    float ss = 0.0f;
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        const float xv = xr[i];
+        float yv;
+        if (a.y) yv = a.y[(long long)r * a.width + i];
+        else
+        {
+            yv = 0.0f;
+            for (int k = 0; k < a.top; k++)
+            {
+                const int e = a.moe_ids[r * a.top + k];
+                const float src = e >= a.n_real ? xv : a.moe_y[((long long)r * a.top + k) * a.width + i];
+                yv = fmaf(a.moe_w[r * a.top + k], src, yv);
+            }
+        }
+        const float s = fmaf(a.alpha, xv, yv);
+        v[i] = s;
+        ss = fmaf(s, s, ss);
+    }
+    ss = block_sum_256(ss, part);
+    const float rinv = 1.0f / sqrtf(ss / (float)a.width + a.eps);
+    T* xh = (T*)a.xh;
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        const float o = v[i] * rinv * (1.0f + ro_ld<T>((const T*)a.w + i));
+        xr[i] = o;
+        if (xh && (void*)xh != (void*)a.x) ro_st<T>(xh + (long long)r * a.width + i, o);
+    }
+}
+
+// ---- router -----------------------------------------------------------------------------------------------------------------
+// One wave per token.  logits fp32 [rows, n_total]; scores = softmax over all n_total; the `top` largest (score + correction) win
+// (first index on a tie); weight = score / (sum of the chosen scores + 1e-20) * scale.
+
+#define ROUTE_MAX_PER_LANE 8
+
+KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const float* correction, int* ids, float* wts,
+                                                    int n_total, int top, float scale)
+{
+    const int r = bid_x();
+    const int lane = lane_id();
+    float s[ROUTE_MAX_PER_LANE], c[ROUTE_MAX_PER_LANE];
+    float mx = -INFINITY;
+    #pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
+    {
+        const int e = lane + 64 * i;
+        s[i] = e < n_total ? logits[(long long)r * n_total + e] : -INFINITY;
+        mx = fmaxf(mx, s[i]);
+    }
+    mx = wave_allreduce_max(mx);
+    float sum = 0.0f;
+    #pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
+    {
+        const int e = lane + 64 * i;
+        s[i] = e < n_total ? expf(s[i] - mx) : 0.0f;
+        sum += s[i];
+    }
+    sum = wave_allreduce_add(sum);
+    #pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
+    {
+        const int e = lane + 64 * i;
+        s[i] = s[i] / sum;
+        c[i] = e < n_total ? s[i] + (correction ? correction[e] : 0.0f) : -INFINITY;
+    }
+    float chosen_sum = 0.0f;
+    float my_w = 0.0f; int my_id = 0;                    // lane k keeps the k-th choice (top <= 64)
+    for (int k = 0; k < top; k++)
+    {
+        float best = -INFINITY; int best_e = 0x7fffffff;
+        #pragma unroll
+        for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
+        {
+            const int e = lane + 64 * i;
+            if (c[i] > best) { best = c[i]; best_e = e; }          // ascending e within a lane: the first maximum stays
+        }
+        const float wbest = wave_allreduce_max(best);
+        int cand = best == wbest ? best_e : 0x7fffffff;
+        #pragma unroll
+        for (int m = 1; m < 64; m <<= 1) cand = min(cand, (int)shfl_xor_u32((u32)cand, m));
+        // the owner hands out the score and retires the expert
+        float sc = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
+            if (lane + 64 * i == cand) { sc = s[i]; c[i] = -INFINITY; }
+        sc = wave_allreduce_add(sc);
+        chosen_sum += sc;
+        if (lane == k) { my_w = sc; my_id = cand; }
+    }
+    if (lane < top)
+    {
+        ids[r * top + lane] = my_id;
+        wts[r * top + lane] = my_w / (chosen_sum + 1e-20f) * scale;
+    }
+}
+
+// per-expert row lists for the grouped linear: thread e scans all (token, choice) pairs in order (deterministic lists)
+KERNEL void __launch_bounds__(256) moe_group_kernel(const int* ids, int pairs, int n_real, int* count, int* offset, int* rows)
+{
+    SHARED int cnt[256];
+    SHARED int off[256];
+    const int e = tid();
+    int c = 0;
+    if (e < n_real)
+        for (int p = 0; p < pairs; p++) c += ids[p] == e;
+    cnt[e] = e < n_real ? c : 0;
+    block_sync();
+    if (e == 0)
+    {
+        int run = 0;
+        for (int i = 0; i < n_real; i++) { off[i] = run; run += cnt[i]; }
+    }
+    block_sync();
+    if (e < n_real)
+    {
+        count[e] = cnt[e]; offset[e] = off[e];
+        int w = off[e];
+        for (int p = 0; p < pairs; p++)
+            if (ids[p] == e) rows[w++] = p;
+    }
+}
+
+// ---- C ABI --------------------------------------------------------------------------------------------------------------------
+
+extern "C" int exl2_embed_scale(const void* table, const int* ids, float* x32, void* xh, int dtype, int rows, int width, int vocab,
+                                float scale, void* stream)
+{
+    EXL2_REQUIRE(table && ids && x32, "embed_scale: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "embed_scale: dtype must be 0 (bfloat16) or 1 (float32)");
+    if (rows <= 0) return EXL2_OK;
+    if (dtype == 0) LAUNCH(embed_scale_kernel<u16>, dim3(rows), dim3(256), 0, stream, (const u16*)table, ids, x32, (u16*)xh, width, vocab, scale);
+    else LAUNCH(embed_scale_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table, ids, x32, (float*)xh, width, vocab, scale);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_rms_rows(const float* x, int ldx, const void* w, int one_plus, void* y, int ldy, int y_f32, const int* row_idx,
+                             int dtype, int rows, int dim, float eps, void* stream)
+{
+    EXL2_REQUIRE(x && w && y, "rms_rows: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "rms_rows: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(dim > 0 && ldx >= dim && ldy >= dim, "rms_rows: bad shape");
+    if (rows <= 0) return EXL2_OK;
+    if (dtype == 0) LAUNCH(rms_rows_kernel<u16>, dim3(rows), dim3(256), 0, stream, x, ldx, (const u16*)w, one_plus, y, ldy, y_f32, row_idx, dim, eps);
+    else LAUNCH(rms_rows_kernel<float>, dim3(rows), dim3(256), 0, stream, x, ldx, (const float*)w, one_plus, y, ldy, 1, row_idx, dim, eps);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_post_norm(float* x, void* xh, const float* y, const void* w, int dtype, int rows, int width, float alpha, float eps,
+                              const float* moe_y, const int* moe_ids, const float* moe_w, int top, int n_real, void* stream)
+{
+    EXL2_REQUIRE(x && w, "post_norm: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "post_norm: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(y || (moe_ids && moe_w && top > 0), "post_norm: neither a sublayer output nor an expert mixture");
+    EXL2_REQUIRE(y || moe_y || n_real == 0, "post_norm: expert outputs missing");
+    EXL2_REQUIRE(width > 0 && (size_t)width * 4 <= 160 * 1024 - 64, "post_norm: row of %d values does not fit the LDS", width);
+    if (rows <= 0) return EXL2_OK;
+    PostNormArgs a;
+    a.x = x; a.xh = xh; a.y = y; a.w = w; a.width = width; a.alpha = alpha; a.eps = eps;
+    a.moe_y = moe_y; a.moe_ids = moe_ids; a.moe_w = moe_w; a.top = top; a.n_real = n_real;
+    const size_t smem = (size_t)width * 4;
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)post_norm_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)post_norm_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    if (dtype == 0) LAUNCH(post_norm_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
+    else LAUNCH(post_norm_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_moe_route_scored(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
+                                     float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, void* stream)
+{
+    EXL2_REQUIRE(logits && ids && wts, "moe_route_scored: null operand");
+    EXL2_REQUIRE(n_total > 0 && n_total <= 64 * ROUTE_MAX_PER_LANE, "moe_route_scored: %d experts (at most %d)", n_total, 64 * ROUTE_MAX_PER_LANE);
+    EXL2_REQUIRE(top > 0 && top <= 64 && top <= n_total, "moe_route_scored: top %d of %d", top, n_total);
+    EXL2_REQUIRE(n_real >= 0 && n_real <= n_total, "moe_route_scored: %d experts with weights of %d", n_real, n_total);
+    if (rows <= 0) return EXL2_OK;
+    LAUNCH(moe_route_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, ids, wts, n_total, top, scale);
+    if (grp_count)
+    {
+        EXL2_REQUIRE(grp_offset && grp_rows, "moe_route_scored: grouped lists need offsets and rows");
+        EXL2_REQUIRE(n_real <= 256, "moe_route_scored: grouped lists for at most 256 experts");
+        LAUNCH(moe_group_kernel, dim3(1), dim3(256), 0, stream, (const int*)ids, rows * top, n_real, grp_count, grp_offset, grp_rows);
+    }
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}

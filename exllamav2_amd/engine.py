@@ -1,0 +1,120 @@
+"""The serving loop over a paged cache: admission, page and slot bookkeeping, batching of unequal requests, sampling.
+
+`Engine.step(entries)` is the one step function: every entry is (request id, its next tokens, places whose logits are wanted);
+all entries of a step are one batch -- portions of prompts beside single decoded tokens -- flattened into rows that carry their
+sequence slot and position, so a position's logits do not depend on how its request was cut into steps or on what else ran
+beside it.  `Generator` drives the same step for generation: prompts are fed in portions while other requests decode,
+tokens are chosen by the library's device sampler."""
+from __future__ import annotations
+
+import random
+
+import torch
+
+from .cache import PAGE_SIZE, PagePool
+from .layered import StepBatch
+
+
+class Engine:
+    def __init__(self, model, max_tokens: int, max_seqs: int = 4, page_size: int = PAGE_SIZE):
+        """The pool is made for `max_tokens` live tokens over at most `max_seqs` live requests, each holding whole pages."""
+        self.model = model
+        pages = -(-int(max_tokens) // page_size) + max_seqs
+        self.pool = PagePool(pages, page_size, max_seqs, model.device)
+        self.cache = model.make_cache(self.pool)
+        self.slots = {}                                           # request id -> slot
+
+    def live(self):
+        return list(self.slots)
+
+    def length(self, rid) -> int:
+        return self.pool.seq_len[self.slots[rid]]
+
+    def step(self, entries, end=()):
+        """entries: iterable of (request id, tokens, want) -- `want` = indices into `tokens` whose logits are returned, in the order
+        of the entries and of `want`.  A request is admitted at its first entry.  `end`: requests whose pages and slot are given
+        back after the step.  Returns fp32 logits [n wanted, vocab] on the device, or None."""
+        ids, seq, pos, want_rows = [], [], [], []
+        seen = set()
+        for rid, tokens, want in entries:
+            if rid in seen:
+                raise RuntimeError(f"request {rid!r} appears twice in one step")
+            seen.add(rid)
+            n = len(tokens)
+            if n == 0:
+                continue
+            if rid not in self.slots:
+                self.slots[rid] = self.pool.open()
+            slot = self.slots[rid]
+            start = self.pool.extend(slot, n)
+            base = len(ids)
+            ids.extend(int(t) for t in tokens)
+            seq.extend([slot] * n)
+            pos.extend(range(start, start + n))
+            for w in want:
+                if not 0 <= w < n:
+                    raise RuntimeError(f"request {rid!r}: wanted place {w} outside its {n} tokens")
+                want_rows.append(base + w)
+        logits = None
+        if ids:
+            dev = self.model.device
+            packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
+            lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
+            batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows))
+            logits = self.model.step(batch, self.cache)
+        for rid in end:
+            self.finish(rid)
+        return logits
+
+    def finish(self, rid) -> None:
+        slot = self.slots.pop(rid, None)
+        if slot is not None:
+            self.pool.close(slot)
+
+
+class Generator:
+    """Continuous batching over Engine.step: up to the pool's slot count of requests are live; a request's prompt is fed in
+    portions of at most `chunk` tokens beside the single tokens of requests that already decode; the next token of a row comes
+    from the library's device sampler (csrc/sampling.hip; temperature 0 = greedy)."""
+
+    def __init__(self, engine: Engine, chunk: int = 512):
+        self.engine, self.chunk = engine, chunk
+
+    def generate(self, prompts, max_new_tokens: int, temperature: float = 0.0, top_k: int = 1, top_p: float = 0.0,
+                 min_p: float = 0.0, seed: int = 0, stop_token: int | None = None):
+        """prompts: list of token-id lists; returns the list of generated token lists (greedy by default)"""
+        eng, ext = self.engine, self.engine.model.ext
+        rng = random.Random(seed)
+        waiting = list(range(len(prompts)))[::-1]
+        state = {}                                               # request -> [tokens not yet fed, generated]
+        out = [[] for _ in prompts]
+        dev, vocab = eng.model.device, eng.model.vocab
+        while waiting or state:
+            while waiting and len(state) < eng.pool.max_seqs:
+                r = waiting.pop()
+                if not prompts[r]:
+                    raise RuntimeError("generate: empty prompt")
+                state[r] = [list(prompts[r]), 0]
+            entries, sampled = [], []
+            for r, (todo, _n) in state.items():
+                part = todo[:self.chunk]
+                del todo[:len(part)]
+                last = not todo
+                entries.append((r, part, [len(part) - 1] if last else []))
+                if last:
+                    sampled.append(r)
+            logits = eng.step(entries)
+            if not sampled:
+                continue
+            toks = torch.empty((len(sampled),), dtype=torch.int32, device=dev)
+            probs = torch.empty((len(sampled),), dtype=torch.float32, device=dev)
+            ext.sample_rows(logits, temperature, top_k, top_p, min_p, rng.random(), toks, probs, vocab=vocab)
+            for r, t in zip(sampled, toks.cpu().tolist()):
+                out[r].append(int(t))
+                state[r][1] += 1
+                if state[r][1] >= max_new_tokens or (stop_token is not None and t == stop_token):
+                    eng.finish(r)
+                    del state[r]
+                else:
+                    state[r][0] = [int(t)]
+        return out

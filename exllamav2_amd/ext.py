@@ -775,6 +775,97 @@ class ExtC:
     def add_i32_(self, t, value: int) -> None:
         self.lib.check(self.lib.exl2_add_i32(self._ptr(t, torch.int32, "t"), t.numel(), int(value), self._stream(t)))
 
+    # ---- unquantized models: dense linears, row-wise steps, latent attention (csrc/dense.hip, rowops.hip, latent_attn.hip) ------
+
+    EPI_NONE, EPI_MUL_SIGMOID_AUX, EPI_SILU_AUX_MUL, EPI_CLAMPED_GLU = 0, 1, 2, 3
+
+    @staticmethod
+    def _dense_code(dtype) -> int:
+        if dtype is torch.bfloat16:
+            return 0
+        if dtype is torch.float32:
+            return 1
+        raise RuntimeError(f"dense operands are bfloat16 or float32, got {dtype}")
+
+    def dense_linear(self, x, w, y, M: int, N: int, K: int, ldx: int, ldw: int, ldy: int, aux=None, ldaux: int = 0, batch: int = 1,
+                     sxb: int = 0, swb: int = 0, syb: int = 0, sauxb: int = 0, w_sel=None, n_sel: int = 0, groups=None,
+                     x_div: int = 1, epi: int = 0, limit: float = 0.0, x_off: int = 0, y_off: int = 0, aux_off: int = 0) -> None:
+        """y = epilogue(x . w^T) on explicit shapes and strides (include/exl2_hip.h: exl2_dense_linear).  x / y / aux may be
+        views INTO larger buffers: *_off are element offsets of the first value.  groups = (count, offset, rows) int32 tensors."""
+        code = self._dense_code(w.dtype)
+        if x.dtype is not w.dtype:
+            raise RuntimeError(f"dense_linear: x is {x.dtype}, w is {w.dtype}")
+        if y.dtype is not w.dtype and y.dtype is not torch.float32:
+            raise RuntimeError(f"dense_linear: y must be {w.dtype} or float32, got {y.dtype}")
+        if batch == 1 and w_sel is None and groups is None and w.numel() < (N - 1) * ldw + K:
+            raise RuntimeError("dense_linear: weight smaller than N x K")
+        gc, go, gr = groups if groups is not None else (None, None, None)
+        self.lib.check(self.lib.exl2_dense_linear(
+            self._ptr(x, None, "x") + x_off * x.element_size(), self._ptr(w, None, "w"),
+            self._ptr(y, None, "y") + y_off * y.element_size(),
+            None if aux is None else self._ptr(aux, torch.float32, "aux") + aux_off * 4, code, int(y.dtype is torch.float32),
+            int(M), int(N), int(K), int(ldx), int(ldw), int(ldy), int(ldaux), int(batch), int(sxb), int(swb), int(syb), int(sauxb),
+            self._ptr(w_sel, torch.int32, "w_sel"), int(n_sel), self._ptr(gc, torch.int32, "grp_count"),
+            self._ptr(go, torch.int32, "grp_offset"), self._ptr(gr, torch.int32, "grp_rows"), int(x_div), int(epi), float(limit),
+            self._stream(y)))
+
+    def embed_scale(self, table, ids, x32, xh, scale: float) -> None:
+        rows, width = ids.numel(), table.shape[1]
+        self.lib.check(self.lib.exl2_embed_scale(self._ptr(table, None, "table"), self._ptr(ids, torch.int32, "ids"),
+                                                 self._ptr(x32, torch.float32, "x32"), self._ptr(xh, table.dtype, "xh"),
+                                                 self._dense_code(table.dtype), rows, width, table.shape[0], float(scale),
+                                                 self._stream(x32)))
+
+    def rms_rows(self, x, ldx: int, w, one_plus: bool, y, ldy: int, rows: int, dim: int, eps: float, row_idx=None, x_off: int = 0) -> None:
+        """y[r, :dim] = rms_norm(x[(row_idx[r] | r), x_off : x_off + dim]) * (w | 1 + w); x fp32, y in w's dtype or fp32"""
+        self.lib.check(self.lib.exl2_rms_rows(self._ptr(x, torch.float32, "x") + x_off * 4, int(ldx), self._ptr(w, None, "w"), int(one_plus),
+                                              self._ptr(y, None, "y"), int(ldy), int(y.dtype is torch.float32),
+                                              self._ptr(row_idx, torch.int32, "row_idx"), self._dense_code(w.dtype), int(rows), int(dim),
+                                              float(eps), self._stream(y)))
+
+    def post_norm(self, x32, xh, y, w, rows: int, alpha: float, eps: float, moe=None) -> None:
+        """x32 <- rms_norm(alpha x32 + y) (1 + w) in place (+ operand copy xh); moe = (expert_out fp32 [rows * top, width] | None,
+        ids int32 [rows, top], weights fp32 [rows, top], n_real) replaces y by the weighted expert mixture"""
+        width = w.numel()
+        my, mi, mw, top, n_real = (None, None, None, 0, 0)
+        if moe is not None:
+            my, mi, mw, n_real = moe
+            top = mi.shape[-1]
+        self.lib.check(self.lib.exl2_post_norm(self._ptr(x32, torch.float32, "x32"), self._ptr(xh, None, "xh"),
+                                               self._ptr(y, torch.float32, "y"), self._ptr(w, None, "w"), self._dense_code(w.dtype),
+                                               int(rows), int(width), float(alpha), float(eps), self._ptr(my, torch.float32, "moe_y"),
+                                               self._ptr(mi, torch.int32, "moe_ids"), self._ptr(mw, torch.float32, "moe_w"),
+                                               int(top), int(n_real), self._stream(x32)))
+
+    def moe_route_scored(self, logits, correction, ids, wts, rows: int, n_total: int, top: int, scale: float, n_real: int,
+                         groups=None) -> None:
+        gc, go, gr = groups if groups is not None else (None, None, None)
+        self.lib.check(self.lib.exl2_moe_route_scored(self._ptr(logits, torch.float32, "logits"),
+                                                      self._ptr(correction, torch.float32, "correction"),
+                                                      self._ptr(ids, torch.int32, "ids"), self._ptr(wts, torch.float32, "wts"),
+                                                      int(rows), int(n_total), int(top), float(scale), int(n_real),
+                                                      self._ptr(gc, torch.int32, "grp_count"), self._ptr(go, torch.int32, "grp_offset"),
+                                                      self._ptr(gr, torch.int32, "grp_rows"), self._stream(logits)))
+
+    def latent_append(self, dkv, ld: int, norm_w, eps: float, rows: int, kv_rank: int, rot: int, rot_dims: int, inv_freq, row_seq,
+                      row_pos, block_table, page: int, cache, dkv_off: int = 0) -> None:
+        self.lib.check(self.lib.exl2_latent_append(self._ptr(dkv, torch.float32, "dkv") + dkv_off * 4, int(ld), self._ptr(norm_w, cache.dtype, "norm_w"),
+                                                   float(eps), self._dense_code(cache.dtype), int(rows), int(kv_rank), int(rot),
+                                                   int(rot_dims), self._ptr(inv_freq, torch.float32, "inv_freq"),
+                                                   self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+                                                   self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page),
+                                                   self._ptr(cache, None, "cache"), self._stream(cache)))
+
+    def latent_attn(self, q, ldq: int, q_head_stride: int, q_rot_off: int, q_abs, cache, page: int, row_seq, row_pos, block_table, out,
+                    rows: int, heads: int, kv_rank: int, rot: int, rot_dims: int, inv_freq, scale: float, window: int) -> None:
+        self.lib.check(self.lib.exl2_latent_attn(self._ptr(q, cache.dtype, "q"), int(ldq), int(q_head_stride), int(q_rot_off),
+                                                 self._ptr(q_abs, torch.float32, "q_abs"), self._ptr(cache, None, "cache"), int(page),
+                                                 self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+                                                 self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1],
+                                                 self._ptr(out, cache.dtype, "out"), self._dense_code(cache.dtype), int(rows), int(heads),
+                                                 int(kv_rank), int(rot), int(rot_dims), self._ptr(inv_freq, torch.float32, "inv_freq"),
+                                                 float(scale), int(window), self._stream(out)))
+
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))
 

@@ -1,0 +1,153 @@
+"""Config-driven decoder stack over unquantized weights: each layer is a mixer and an optional feed-forward taken from two
+registries, joined by post-norm residual steps  x <- norm(alpha x + sublayer(x)) (1 + w)  on an fp32 residual stream.
+
+The model has ONE forward, `step(batch, cache)`: the rows of a step are a flat list of tokens, each with its sequence slot and
+position, so whole prompts, portions of prompts and single decoded tokens of several requests run through the same launches
+(exllamav2_amd.engine builds the batches).  Operand dtype bfloat16 (weights, linear inputs, cache rows; fp32 accumulation) or
+float32 (everything in true 32-bit); norms, softmax, routing, rotation and the residual stream are fp32 in both."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .cache import LatentCache, PagePool
+from .config import LayeredConfig
+from .dense_linear import DenseLinear
+from .ext import ext_c
+from .latent_attn import LatentAttention
+from .mlp import DenseGatedMLP
+from .moe_mlp import ScoredMoEMLP
+from .rmsnorm import PostNorm
+
+
+def _latent_attention(model, key, idx, spec):
+    m = spec["mixer"]
+    return LatentAttention(model, key, idx, heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                           kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), window=int(m["mask"]["size"]),
+                           rot_base=float(m["rot"]["base"]), rot_dims=int(m["rot"]["dims"]), scale=float(m["scale"]),
+                           kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None))
+
+
+def _dense_mlp(model, key, idx, spec):
+    return DenseGatedMLP(model, key, idx)
+
+
+def _moe_mlp(model, key, idx, spec):
+    r, e = spec["router"], spec["expert"]
+    return ScoredMoEMLP(model, key, idx, experts=int(r["experts"]), identity=int(r.get("identity", 0)), top=int(r["top"]),
+                        route_scale=float(r["scale"]), ff=int(e["ff"]), limit=float(e["limit"]))
+
+
+MIXERS = {"latent_attention": _latent_attention}             # config `type` -> builder(model, key, layer index, layer spec)
+FEED_FORWARDS = {"dense": _dense_mlp, "moe": _moe_mlp}       # config `mlp.kind` -> builder(model, key, layer index, mlp spec)
+
+
+@dataclass
+class StepBatch:
+    """Device-side description of one step: int32 tensors ids / row_seq / row_pos [rows], block_table [slots, pages],
+    logit_rows [n_logits] (rows whose logits are wanted)."""
+    ids: torch.Tensor
+    row_seq: torch.Tensor
+    row_pos: torch.Tensor
+    block_table: torch.Tensor
+    logit_rows: torch.Tensor
+    rows: int
+    n_logits: int
+
+
+class LayeredModel:
+    def __init__(self, config: LayeredConfig, device="cuda:0", dtype=torch.bfloat16, ext=None):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise RuntimeError("LayeredModel: operand dtype is bfloat16 or float32")
+        self.config, self.device, self.dtype, self.ext = config, torch.device(device), dtype, ext or ext_c
+        self.width, self.vocab, self.norm_eps = config.width, config.vocab, config.norm_eps
+        self.layers = []
+        self.loaded = False
+
+    # ---- loading --------------------------------------------------------------------------------------------------------------
+
+    def load(self, tensors: dict):
+        """tensors: name -> device tensor as stored (bfloat16 weights); converted once to the operand dtype"""
+        cfg = self.config
+        conv = lambda t: t.to(self.dtype).contiguous() if t.is_floating_point() else t
+
+        def need(name):
+            if name not in tensors:
+                raise RuntimeError(f"checkpoint has no tensor '{name}'")
+            return conv(tensors[name])
+
+        self.embed = need("embed")
+        if tuple(self.embed.shape) != (cfg.vocab, cfg.width):
+            raise RuntimeError(f"embed is {tuple(self.embed.shape)}, config says {(cfg.vocab, cfg.width)}")
+        self.layers = []
+        for i, spec in enumerate(cfg.layers):
+            key = f"l{i}"
+            if spec["type"] not in MIXERS:
+                raise RuntimeError(f"layer {i}: unknown mixer type '{spec['type']}' (known: {sorted(MIXERS)})")
+            mixer = MIXERS[spec["type"]](self, key, i, spec).load(lambda n, k=key: need(f"{k}.mix.{n}"))
+            norm1 = PostNorm(self.ext, key + ".norm1", need(key + ".norm1"), cfg.norm_eps, cfg.postln_alpha)
+            ff, norm2 = None, None
+            ms = spec.get("mlp")
+            if ms is not None:
+                if ms["kind"] not in FEED_FORWARDS:
+                    raise RuntimeError(f"layer {i}: unknown feed-forward kind '{ms['kind']}' (known: {sorted(FEED_FORWARDS)})")
+                ff = FEED_FORWARDS[ms["kind"]](self, key + ".mlp", i, ms).load(lambda n, k=key: need(f"{k}.mlp.{n}"))
+            if ff is not None or key + ".norm2" in tensors:
+                norm2 = PostNorm(self.ext, key + ".norm2", need(key + ".norm2"), cfg.norm_eps, cfg.postln_alpha)
+            self.layers.append((mixer, norm1, ff, norm2))
+        for i, (mixer, *_rest) in enumerate(self.layers):
+            j = getattr(mixer, "kv_from", None)
+            if j is not None:
+                if not (0 <= j < len(self.layers)) or getattr(self.layers[j][0], "kv_from", 0) is not None:
+                    raise RuntimeError(f"layer {i}: kv_from {j} does not name a layer with keys and values of its own")
+                src = self.layers[j][0]
+                if (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
+                    raise RuntimeError(f"layer {i}: its latent sizes / rotation differ from layer {j}'s, whose cache it reads")
+        self.final_norm = need("final.norm")
+        self.head = DenseLinear(self.ext, "head", need("head"))
+        self.loaded = True
+        return self
+
+    def weight_bytes(self) -> int:
+        n = self.head.weight_bytes()
+        for mixer, _n1, ff, _n2 in self.layers:
+            n += mixer.weight_bytes() + (ff.weight_bytes() if ff is not None else 0)
+        return n
+
+    # ---- cache ----------------------------------------------------------------------------------------------------------------
+
+    def make_cache(self, pool: PagePool) -> LatentCache:
+        widths, owner = {}, {}
+        for i, (mixer, *_rest) in enumerate(self.layers):
+            if mixer.kv_from is None:
+                widths[i] = mixer.cache_row_width
+                owner[i] = i
+            else:
+                owner[i] = mixer.kv_from
+        return LatentCache(pool, widths, owner, self.dtype)
+
+    # ---- forward ----------------------------------------------------------------------------------------------------------------
+
+    def step(self, batch: StepBatch, cache) -> torch.Tensor | None:
+        """Runs the batch's rows through all layers, appending to the cache; returns fp32 logits [n_logits, vocab] (None if
+        no row wants them)."""
+        ext, cfg, rows = self.ext, self.config, batch.rows
+        x32 = torch.empty((rows, self.width), dtype=torch.float32, device=self.device)
+        xh = x32 if self.dtype is torch.float32 else torch.empty((rows, self.width), dtype=self.dtype, device=self.device)
+        ext.embed_scale(self.embed, batch.ids, x32, xh, cfg.embedding_scale)
+        for mixer, norm1, ff, norm2 in self.layers:
+            y = mixer.forward(xh, rows, batch, cache)
+            norm1.forward(x32, xh, y, rows)
+            if norm2 is not None:
+                if ff is None:
+                    y, mix = torch.zeros_like(x32), None
+                else:
+                    y, mix = ff.forward(xh, rows)
+                norm2.forward(x32, xh, y, rows, moe=mix)
+        if batch.n_logits == 0:
+            return None
+        xn = torch.empty((batch.n_logits, self.width), dtype=self.dtype, device=self.device)
+        ext.rms_rows(x32, self.width, self.final_norm, True, xn, self.width, batch.n_logits, self.width, cfg.norm_eps,
+                     row_idx=batch.logit_rows)
+        return self.head.forward(xn, batch.n_logits, out_dtype=torch.float32)

@@ -39,3 +39,27 @@ class ExLlamaV2MLP:
         row pre-pass + dequantize-into-MFMA GEMMs, csrc/modules.hip:exl2_q_mlp_forward)."""
         self.ext.q_mlp_forward_(self.q_handle, hidden_states)
         return hidden_states
+
+
+class DenseGatedMLP:
+    """Gated MLP over unquantized weights: W_down(silu(W_gate h) * (W_up h)) in three launches -- the activation and the product
+    run in the up projection's epilogue (csrc/dense.hip).  Returns the sublayer's output in fp32; the residual step is the
+    caller's (pre- or post-norm)."""
+
+    def __init__(self, model, key: str, layer_idx: int):
+        self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
+
+    def load(self, get):
+        from .dense_linear import DenseLinear
+        self.gate = DenseLinear(self.ext, self.key + ".gate", get("gate"))
+        self.up = DenseLinear(self.ext, self.key + ".up", get("up"))
+        self.down = DenseLinear(self.ext, self.key + ".down", get("down"))
+        return self
+
+    def weight_bytes(self) -> int:
+        return self.gate.weight_bytes() + self.up.weight_bytes() + self.down.weight_bytes()
+
+    def forward(self, xh: torch.Tensor, rows: int):
+        g = self.gate.forward(xh, rows, out_dtype=torch.float32)
+        a = self.up.forward(xh, rows, aux=g, aux_ld=g.shape[-1], epi=self.ext.EPI_SILU_AUX_MUL)
+        return self.down.forward(a, rows, out_dtype=torch.float32), None

@@ -50,3 +50,73 @@ class ExLlamaV2MoEMLP:
         h = hidden_states.shape[-1]
         self.ext.q_moe_mlp_forward_(self.q_handle, hidden_states.view(-1, h))
         return hidden_states
+
+
+class ScoredMoEMLP:
+    """Sparse MoE over unquantized experts with a score-corrected router and identity experts.
+
+    Router: logits in fp32, scores = softmax over ALL router outputs; the `top` largest (score + correction) are chosen, their
+    weights are the uncorrected scores divided by their sum, times `route_scale`.  The last `identity` router outputs are experts
+    without tensors whose output is the token itself.  A real expert is the clamped gated unit
+    W_down(g sigmoid(1.702 g) (u + 1)), g = min(W_gate h, limit), u = clamp(W_up h, +-limit), evaluated in the up projection's
+    epilogue.  Few rows (decoding): every (token, choice) pair is one row that names its expert's slab.  Many rows: the pairs are
+    listed per expert on the device and one grouped launch per projection runs all experts (no host round trip either way).
+    forward returns (None, mixture): the weighted sum is taken inside the residual step's launch (rmsnorm.PostNorm)."""
+
+    PAIR_ROWS_MAX = 64                                   # (token, choice) pairs up to which rows pick their slab individually
+
+    def __init__(self, model, key: str, layer_idx: int, *, experts: int, identity: int, top: int, route_scale: float, ff: int,
+                 limit: float):
+        self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
+        self.experts, self.identity, self.top, self.route_scale, self.ff, self.limit = experts, identity, top, route_scale, ff, limit
+
+    def load(self, get):
+        from .dense_linear import DenseLinear
+        E = self.experts
+        self.router = DenseLinear(self.ext, self.key + ".router", get("router"))
+        if self.router.out_features != E + self.identity:
+            raise RuntimeError(f"{self.key}: router has {self.router.out_features} outputs for {E} + {self.identity} experts")
+        self.correction = get("correction").to(torch.float32).contiguous()
+        if E:
+            stack = lambda name: torch.stack([get(f"e{e}.{name}") for e in range(E)], 0)
+            self.gate = DenseLinear(self.ext, self.key + ".gate", stack("gate"))
+            self.up = DenseLinear(self.ext, self.key + ".up", stack("up"))
+            self.down = DenseLinear(self.ext, self.key + ".down", stack("down"))
+        return self
+
+    def weight_bytes(self) -> int:
+        """bytes one token streams: the router and `top` experts (an upper bound when identity experts are chosen)"""
+        n = self.router.weight_bytes()
+        if self.experts:
+            n += (self.gate.weight_bytes() + self.up.weight_bytes() + self.down.weight_bytes()) // self.experts * min(self.top, self.experts)
+        return n
+
+    def forward(self, xh: torch.Tensor, rows: int):
+        ext, m = self.ext, self.model
+        E, top, ff, width = self.experts, self.top, self.ff, m.width
+        dev, dt = m.device, m.dtype
+        n_total = E + self.identity
+        logits = self.router.forward(xh, rows, out_dtype=torch.float32)
+        ids = torch.empty((rows, top), dtype=torch.int32, device=dev)
+        wts = torch.empty((rows, top), dtype=torch.float32, device=dev)
+        pairs = rows * top
+        grouped = pairs > self.PAIR_ROWS_MAX and E > 0
+        groups = None
+        if grouped:
+            groups = (torch.empty((E,), dtype=torch.int32, device=dev), torch.empty((E,), dtype=torch.int32, device=dev),
+                      torch.empty((pairs,), dtype=torch.int32, device=dev))
+        ext.moe_route_scored(logits, self.correction, ids, wts, rows, n_total, top, self.route_scale, E, groups=groups)
+        if E == 0:
+            return None, (None, ids, wts, 0)
+        g = torch.empty((pairs, ff), dtype=torch.float32, device=dev)
+        a = torch.empty((pairs, ff), dtype=dt, device=dev)
+        y = torch.empty((pairs, width), dtype=torch.float32, device=dev)
+        if grouped:
+            kw = dict(batch=E, groups=groups)
+        else:
+            kw = dict(w_sel=ids.view(-1), n_sel=E)
+        ext.dense_linear(xh, self.gate.weight, g, pairs, ff, width, width, width, ff, swb=ff * width, x_div=top, **kw)
+        ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=top,
+                         aux=g, ldaux=ff, epi=ext.EPI_CLAMPED_GLU, limit=self.limit, **kw)
+        ext.dense_linear(a, self.down.weight, y, pairs, width, ff, ff, ff, width, swb=width * ff, **kw)
+        return None, (y, ids, wts, E)

@@ -24,3 +24,15 @@ class ExLlamaV2RMSNorm:
         hidden_states = hidden_states * torch.rsqrt(variance + self.variance_epsilon)
         hidden_states = hidden_states.to(self.weight.dtype)
         return hidden_states * self.weight
+
+
+class PostNorm:
+    """The residual step of a post-norm layer, x <- rms_norm(alpha x + sublayer(x)) (1 + w), as ONE launch in place on the fp32
+    residual stream (csrc/rowops.hip: post_norm_kernel); it also leaves the operand-dtype copy the next linears read.  The weight is
+    stored around zero.  `moe` routes the mixture of a token's chosen experts (identity experts included) through the same launch."""
+
+    def __init__(self, ext, key: str, weight: torch.Tensor, eps: float, alpha: float):
+        self.ext, self.key, self.weight, self.eps, self.alpha = ext, key, weight.contiguous(), eps, alpha
+
+    def forward(self, x32: torch.Tensor, xh, y, rows: int, moe=None) -> None:
+        self.ext.post_norm(x32, xh, y, self.weight, rows, self.alpha, self.eps, moe=moe)

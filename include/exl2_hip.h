@@ -381,6 +381,51 @@ int exl2_graph_end_capture(void* stream, void** graph_exec);
 int exl2_graph_launch(void* graph_exec, void* stream);
 int exl2_graph_free(void* graph_exec);
 
+/* ---- unquantized models: dense linears, row-wise steps, latent attention (csrc/dense.hip, rowops.hip, latent_attn.hip) ------
+   dtype: 0 = bfloat16 operands (weights, activations fed to a linear, cache rows), 1 = float32 (true 32-bit arithmetic, no
+   reduced-precision matrix mode).  Accumulation, norms, softmax, routing, rotation and the residual stream are fp32 in both. */
+
+/* y[r, n] = epilogue(sum_k x[r, k] w[n, k]); w is [N, K] with leading dimension ldw.  batch > 1: blockIdx.z batches with element
+   offsets sxb / swb / syb / sauxb per batch.  w_sel (nullable): int32 [M], row r multiplies slab w_sel[r] (offset w_sel[r] * swb);
+   rows whose entry is outside [0, n_sel) are left untouched.  grp_* (nullable): grouped form, batch z multiplies rows
+   grp_rows[grp_offset[z] .. + grp_count[z]) (M = the largest possible count).  Row p reads x row p / x_div.  epi: 0 none,
+   1 acc * sigmoid(aux), 2 silu(aux) * acc, 3 min(aux, limit) * sigmoid(1.702 min(aux, limit)) * (clamp(acc, +-limit) + 1);
+   aux fp32 with ldaux, indexed like y.  y_f32: the result is stored as fp32 (always with dtype 1). */
+int exl2_dense_linear(const void* x, const void* w, void* y, const float* aux, int dtype, int y_f32,
+                      int M, int N, int K, int ldx, int ldw, int ldy, int ldaux,
+                      int batch, long long sxb, long long swb, long long syb, long long sauxb,
+                      const int* w_sel, int n_sel, const int* grp_count, const int* grp_offset, const int* grp_rows,
+                      int x_div, int epi, float limit, void* stream);
+/* x32[r] = table[ids[r]] * scale (fp32 residual stream); xh (nullable): the same rows in the operand dtype */
+int exl2_embed_scale(const void* table, const int* ids, float* x32, void* xh, int dtype, int rows, int width, int vocab,
+                     float scale, void* stream);
+/* y[r, :dim] = x[row_idx ? row_idx[r] : r, :dim] / sqrt(mean(x^2) + eps) * (one_plus ? 1 + w : w); x fp32, y operand dtype or fp32 */
+int exl2_rms_rows(const float* x, int ldx, const void* w, int one_plus, void* y, int ldy, int y_f32, const int* row_idx,
+                  int dtype, int rows, int dim, float eps, void* stream);
+/* the post-norm residual step x <- rms_norm(alpha x + y) (1 + w), in place on the fp32 stream, + the operand-dtype copy xh
+   (nullable).  y == NULL: y = sum_k moe_w[r, k] * (moe_ids[r, k] >= n_real ? x[r] : moe_y[r * top + k]) (expert mixture with
+   identity experts). */
+int exl2_post_norm(float* x, void* xh, const float* y, const void* w, int dtype, int rows, int width, float alpha, float eps,
+                   const float* moe_y, const int* moe_ids, const float* moe_w, int top, int n_real, void* stream);
+/* router: scores = softmax(logits) over n_total; the `top` largest (score + correction) are chosen; weight = score / (sum of the
+   chosen scores + 1e-20) * scale.  ids int32 / wts fp32 [rows, top].  grp_* (nullable): also the per-expert lists of
+   (row * top + k) pairs for experts < n_real, in pair order (the grouped form of exl2_dense_linear). */
+int exl2_moe_route_scored(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
+                          float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, void* stream);
+/* new cache rows: dkv fp32 [rows, ld] = kv_rank latent values (RMS-normed with norm_w) then rot shared key values (the first
+   rot_dims rotated in interleaved pairs by angle pos * inv_freq[i]); row r goes to position row_pos[r] of sequence row_seq[r]:
+   page block_table[row_seq[r] * bt_stride + pos / page] of cache [pages, page, kv_rank + rot]. */
+int exl2_latent_append(const float* dkv, int ld, const void* norm_w, float eps, int dtype, int rows, int kv_rank, int rot,
+                       int rot_dims, const float* inv_freq, const int* row_seq, const int* row_pos, const int* block_table,
+                       int bt_stride, int page, void* cache, void* stream);
+/* sliding-window softmax attention in latent space: out[r, h, :kv_rank] = sum_j p_j c_j over max(0, pos - window + 1) <= j <= pos,
+   score_j = (q_abs[r, h] . c_j + rot(q[r, h, rot part], pos) . k_rot_j) * scale.  q: operand dtype, q_abs fp32 [rows, heads, kv_rank],
+   out operand dtype [rows, heads, kv_rank]. */
+int exl2_latent_attn(const void* q, int ldq, int q_head_stride, int q_rot_off, const float* q_abs, const void* cache, int page,
+                     const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, void* out, int dtype,
+                     int rows, int heads, int kv_rank, int rot, int rot_dims, const float* inv_freq, float scale, int window,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -236,6 +236,42 @@ DEV f32x4 mfma_16x16x32_f16(f16x8 a, f16x8 b, f32x4 c)
     return d;
 }
 
+
+// ---- bfloat16 as its 16 bits + v_mfma_f32_16x16x32_bf16 (hw.h) ---------------------------------------------------------------
+DEV float bf16_to_f32(u16 v) { return as_f32((u32)v << 16); }
+DEV u16 f32_to_bf16(float f)
+{
+    u32 u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (u16)(u >> 16);
+}
+DEV f32x4 mfma_16x16x32_bf16(u32x4 a, u32x4 b, f32x4 c)
+{
+    EmuWave& w = emu_ctx_->wave[wave_id()];
+    const int l = lane_id();
+    memcpy(w.slot[l], &a, 16);
+    memcpy(w.slot[l] + 16, &b, 16);
+    w.bar.wait();
+    const int col = l & 15;
+    f32x4 d = c;
+    for (int r = 0; r < 4; r++)
+    {
+        const int row = (l >> 4) * 4 + r;
+        float acc = d[r];
+        for (int j = 0; j < 4; j++)
+        {
+            u16 av[8], bv[8];
+            memcpy(av, w.slot[row + 16 * j], 16);
+            memcpy(bv, w.slot[col + 16 * j] + 16, 16);
+            for (int e = 0; e < 8; e++) acc += bf16_to_f32(av[e]) * bf16_to_f32(bv[e]);
+        }
+        d[r] = acc;
+    }
+    w.bar.wait();
+    return d;
+}
+
 DEV float dot2_f32_f16(f16x2 a, f16x2 b, float c) { return c + (float)a.x * (float)b.x + (float)a.y * (float)b.y; }
 
 // ds_read_b64_tr_b16 (hw.h): lane 16 g + i gets element (i % 4) of what lanes 16 g + 4 j + i / 4 (j = 0 .. 3) pointed at
