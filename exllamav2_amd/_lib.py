@@ -14,6 +14,8 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # EXL2_HIP_LIB: alternative build of the SAME library (kernel-tuning A/B runs, trace build); never a different backend
 HIP_LIB_PATH = os.environ.get("EXL2_HIP_LIB") or os.path.join(_HERE, "libexl2_hip.so")
+# the subset library of the unquantized models (build.py: DENSE_SOURCES); bound when the whole library has not been built
+HIP_DENSE_LIB_PATH = os.path.join(_HERE, "libexl2_hip_dense.so")
 
 vp = C.c_void_p
 ci = C.c_int
@@ -124,8 +126,15 @@ class Exl2Error(RuntimeError):
     pass
 
 
+def _absent(name: str, path: str):
+    def call(*_a, **_k):
+        raise Exl2Error(f"{name} is not part of {os.path.basename(path)} (the subset built for unquantized models): build the whole "
+                        f"library with `python -c \"import __graft_entry__ as g; g.build()\"`")
+    return call
+
+
 class Lib:
-    def __init__(self, path: str):
+    def __init__(self, path: str, allow_missing: bool = False):
         if not os.path.exists(path):
             raise Exl2Error(
                 f"{path} not found: the HIP library is not built. Run `python -c \"import __graft_entry__ as g; "
@@ -138,13 +147,15 @@ class Lib:
                 fn = getattr(self.dll, name)
             except AttributeError:
                 self.missing.append(name)
+                if allow_missing:
+                    setattr(self, name, _absent(name, path))
                 continue
             fn.restype = res
             fn.argtypes = args
             setattr(self, name, fn)
         # (EXL2_LIB_ALLOW_MISSING=1: bisecting with a library built from an OLDER source state -- tools only; a call of a missing entry
         # point is then an AttributeError)
-        if self.missing and os.environ.get("EXL2_LIB_ALLOW_MISSING", "0") == "0":
+        if self.missing and not allow_missing and os.environ.get("EXL2_LIB_ALLOW_MISSING", "0") == "0":
             raise Exl2Error(f"{path} does not export: {', '.join(self.missing)}")
 
     def last_error(self) -> str:
@@ -165,5 +176,8 @@ def hip_lib() -> Lib:
     if _hip is None:
         with _lock:
             if _hip is None:
-                _hip = Lib(HIP_LIB_PATH)
+                if not os.path.exists(HIP_LIB_PATH) and os.path.exists(HIP_DENSE_LIB_PATH) and "EXL2_HIP_LIB" not in os.environ:
+                    _hip = Lib(HIP_DENSE_LIB_PATH, allow_missing=True)
+                else:
+                    _hip = Lib(HIP_LIB_PATH)
     return _hip

@@ -68,6 +68,12 @@ def read_config(model_dir: str):
     return name, ARCHITECTURES[name][0](d)
 
 
+def needs_whole_library(model_dir: str) -> bool:
+    """False for architectures served by the dense-model subset of the library alone (build.py: DENSE_SOURCES)"""
+    name, _cfg = read_config(model_dir)
+    return ARCHITECTURES[name][1] is not _build_layered
+
+
 def load_model(model_dir: str, device="cuda:0", dtype=None, ext=None):
     from .ext import ext_c
     from .loader import load_tensors

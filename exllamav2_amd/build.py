@@ -9,6 +9,10 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libexl2_hip.so")
+# What the unquantized (dense-weight) models need -- their kernels, the checkpoint reader, the sampler, graphs -- as a library of its
+# own: a fresh checkout that only ever serves such a model compiles these seven sources (about a minute) instead of the whole tree.
+DENSE_SOURCES = ("errors", "dense", "rowops", "latent_attn", "stloader", "sampling", "graph")
+OUT_DENSE = os.path.join(HERE, "libexl2_hip_dense.so")
 
 
 def sources():
@@ -28,9 +32,14 @@ def _obj_dir() -> str:
     return d
 
 
-def build(force: bool = False, verbose: bool = False) -> str:
+def build_dense(force: bool = False, verbose: bool = False) -> str:
+    """The subset library of DENSE_SOURCES (same objects, same flags, its own link)."""
+    return build(force=force, verbose=verbose, only=DENSE_SOURCES, out=OUT_DENSE)
+
+
+def build(force: bool = False, verbose: bool = False, only=None, out: str = OUT) -> str:
     """One object per .hip file (compiled in parallel, re-compiled only when the file or a header is newer), one link."""
-    if not force and not needs_build():
+    if not force and only is None and not needs_build():
         return OUT
     from concurrent.futures import ThreadPoolExecutor
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
@@ -42,6 +51,8 @@ def build(force: bool = False, verbose: bool = False) -> str:
     hdr_time = max(os.path.getmtime(f) for f in headers) if headers else 0.0
     objs, jobs = [], []
     for src in sources():
+        if only is not None and os.path.basename(src)[:-4] not in only:
+            continue
         obj = os.path.join(_obj_dir(), os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
         if force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(src), hdr_time):
@@ -54,8 +65,9 @@ def build(force: bool = False, verbose: bool = False) -> str:
 
     with ThreadPoolExecutor(max_workers=max(1, min(len(jobs), os.cpu_count() or 4))) as ex:
         list(ex.map(run, jobs))
-    run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", OUT] + objs)
-    return OUT
+    run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", out + ".part"] + objs)
+    os.replace(out + ".part", out)
+    return out
 
 
 if __name__ == "__main__":

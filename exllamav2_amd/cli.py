@@ -16,12 +16,19 @@ import os
 import sys
 
 
-def _ensure_built():
-    """first use in a fresh checkout: compile the gfx950 library in-tree"""
-    from . import build
-    if build.needs_build():
+def _ensure_built(model_dir: str):
+    """First use in a fresh checkout: compile in-tree what the model's architecture needs -- the subset library for the
+    unquantized layer stacks, the whole library for the quantized Llama family.  A library that is already there is used as it is."""
+    from . import _lib, build
+    from .architectures import needs_whole_library
+    if os.path.exists(_lib.HIP_LIB_PATH):
+        return
+    if needs_whole_library(model_dir):
         print("building the HIP library (first use) ...", file=sys.stderr, flush=True)
         build.build(verbose=False)
+    elif not os.path.exists(_lib.HIP_DENSE_LIB_PATH):
+        print("building the dense-model subset of the HIP library (first use) ...", file=sys.stderr, flush=True)
+        build.build_dense(verbose=False)
 
 
 def _dtype(name):
@@ -30,7 +37,7 @@ def _dtype(name):
 
 
 def cmd_generate(a) -> int:
-    _ensure_built()
+    _ensure_built(a.model)
     from .architectures import load_model
     from .engine import Engine, Generator
     model = load_model(a.model, device=a.device, dtype=_dtype(a.dtype))
@@ -52,7 +59,7 @@ def cmd_trace(a) -> int:
     if a.dtype not in ("bfloat16", "float32"):
         print("trace: --dtype is bfloat16 or float32", file=sys.stderr)
         return 2
-    _ensure_built()
+    _ensure_built(a.model)
     from .architectures import load_model
     from .engine import Engine
     model = load_model(a.model, device=a.device, dtype=_dtype(a.dtype))

@@ -11,21 +11,7 @@ void qmatrix_destroy(QMatrix* qm);
 int qmatrix_reconstruct(const QMatrix* qm, f16* out, void* stream);
 int qgemv_launch(GemvJob* jobs, int n_jobs, int M, bool gptq, void* stream);
 
-static thread_local char g_err[512] = "";
-
-void exl2_set_error(const char* fmt, ...)
-{
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_err, sizeof(g_err), fmt, ap);
-    va_end(ap);
-}
-
 extern "C" {
-
-const char* exl2_last_error(void) { return g_err; }
-
-int exl2_abi_version(void) { return 1; }
 
 int exl2_make_q_matrix(void** handle, int device, int height, int width, int groups,
                        void* q_weight, void* q_perm, void* q_invperm, void* q_scale, void* q_scale_max, void* q_groups,
