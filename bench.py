@@ -61,6 +61,11 @@ def parse():
     p.add_argument("--windows", type=int, default=5, help="timed windows of --steps steps (each after --warmup untimed steps from the same "
                                                            "cache position); the MEDIAN window is the reported value")
     p.add_argument("--headline-only", action="store_true", help="= --no-cpu-baseline --no-prefill --no-dropin --no-ctx-window (A/B runs)")
+    p.add_argument("--design", default=None, choices=["benolix"],
+                   help="instead of the headline: prefill / decode throughput of the latent-attention layer stack at real layer sizes "
+                        "beside the quantized Mixtral-style stack of equal size (exllamav2_amd/bench_layered.py); one JSON line each")
+    p.add_argument("--design-sizes", default="w2048,w4096")
+    p.add_argument("--design-no-peer", action="store_true", help="--design: skip the quantized peer model")
     a = p.parse_args()
     if a.headline_only:
         a.no_cpu_baseline = a.no_prefill = a.no_dropin = a.no_ctx_window = True
@@ -746,6 +751,11 @@ def spawn_ranks(n: int) -> None:
 
 
 def main():
+    if "--design" in sys.argv:
+        a = parse()
+        from exllamav2_amd import bench_layered
+        bench_layered.run(a.design_sizes.split(","), peer=not a.design_no_peer)
+        return
     args = parse()
     if args.cpu_baseline_only:
         print(json.dumps(cpu_baseline(make_cfg(args.model, 2048), args.recipe)))

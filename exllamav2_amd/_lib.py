@@ -114,6 +114,7 @@ PROTOTYPES = {
     "exl2_moe_route_scored": (ci, [vp, vp, vp, vp, ci, ci, ci, cf, ci, vp, vp, vp, vp]),
     "exl2_latent_append": (ci, [vp, ci, vp, cf, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, ci, vp, vp]),
     "exl2_latent_attn": (ci, [vp, ci, ci, ci, vp, vp, ci, vp, vp, vp, ci, vp, ci, ci, ci, ci, ci, ci, vp, cf, ci, vp]),
+    "exl2_latent_attn_tiles": (ci, [vp, ci, ci, ci, vp, vp, ci, vp, vp, vp, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, ci, ci, vp, cf, ci, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

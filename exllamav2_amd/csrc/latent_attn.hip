@@ -169,6 +169,258 @@ KERNEL void __launch_bounds__(256) latent_attn_kernel(const LatAttnArgs a)
     }
 }
 
+// ---- bfloat16 on the matrix cores ----------------------------------------------------------------------------------------------
+// A wave owns 16 query vectors that share their keys: TR = 16: sixteen consecutive positions of one sequence x one head (a prompt's
+// portion; the four waves of a workgroup take four heads), TR = 1: one position x sixteen heads (a decoded token).  Keys go by in
+// steps of 32: the workgroup stages the step's cache rows in LDS twice -- row-major for S = Q C^T (both operands K-contiguous) and
+// transposed ([latent element][key]) for O += P C, whose B operand wants 8 consecutive KEYS of one latent element per lane.  The
+// scores leave the accumulators through a wave-private LDS tile to become the A operand of the second product.  Softmax state
+// (running maximum, sum) is per query row = per accumulator row, kept in registers; fp32 throughout, P rounded to bfloat16 for the
+// matrix core.  grid.z > 1 splits the key steps over workgroups (decoding against a long window): partial (m, l, O) go to
+// scratch and latent_attn_merge_kernel joins them.
+
+struct LatMfmaArgs
+{
+    const u16* q; int ldq, q_head_stride, q_rot_off;
+    const float* q_abs;
+    const u16* cache; int page;
+    const int* row_seq; const int* row_pos; const int* block_table; int bt_stride;
+    const int* tile_row0; const int* tile_rows;
+    u16* out;
+    float* part_o; float* part_ml; int nsplit;
+    int H, R, rot, rot_dims;
+    const float* inv_freq;
+    float scale; int window;
+    int DP;                                                  // kv_rank + rot rounded up to a multiple of 32
+};
+
+#define LA_KT 32
+#define LA_TS 40                                             // row stride (values) of the transposed and the probability tiles
+#define LA_ROT_STEPS 4
+
+DEV u32 la_pack2(float lo, float hi) { return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16); }
+
+template <int NT, int TR>
+KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
+{
+    DYN_SMEM(smem);
+    const int tile = bid_x(), hb = bid_y(), split = bid_z();
+    const int w = wave_id(), lane = lane_id(), li = lane & 15, g = lane >> 4, t = tid();
+    const int r0 = a.tile_row0[tile];
+    const int n = TR == 16 ? a.tile_rows[tile] : 1;
+    const int p0 = a.row_pos[r0];
+    const int* bt = a.block_table + (long long)a.row_seq[r0] * a.bt_stride;
+    const int H = a.H, R = a.R, D = a.R + a.rot, DP = a.DP, CS = DP + 8;
+    u16* Cs = (u16*)smem;                                    // [32][CS]
+    u16* Ct = Cs + LA_KT * CS;                               // [R][LA_TS]
+    u16* Ps = Ct + R * LA_TS + w * 16 * LA_TS;               // [16][LA_TS], this wave's
+
+    // the query vector this lane feeds as A-operand row li
+    int qrow, qhead;
+    if (TR == 16) { qrow = r0 + min(li, n - 1); qhead = hb * 4 + w; }
+    else { qrow = r0; qhead = (hb * 4 + w) * 16 + li; }
+    const bool wave_live = (TR == 16 ? hb * 4 + w : (hb * 4 + w) * 16) < H;
+    const int qh = min(qhead, H - 1);
+    const int qpos = a.row_pos[qrow];
+
+    constexpr int KSC = NT / 2;
+    u32x4 qf[KSC + LA_ROT_STEPS];
+    {
+        const float* qa = a.q_abs + ((long long)qrow * H + qh) * R;
+        #pragma unroll
+        for (int ks = 0; ks < KSC; ks++)
+        {
+            qf[ks] = (u32x4){0u, 0u, 0u, 0u};
+            if (ks * 32 < R)
+            {
+                const float* s = qa + ks * 32 + 8 * g;
+                qf[ks] = (u32x4){la_pack2(s[0], s[1]), la_pack2(s[2], s[3]), la_pack2(s[4], s[5]), la_pack2(s[6], s[7])};
+            }
+        }
+        const u16* qr = a.q + (long long)qrow * a.ldq + (long long)qh * a.q_head_stride + a.q_rot_off;
+        #pragma unroll
+        for (int ks = 0; ks < LA_ROT_STEPS; ks++)
+        {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (ks * 32 < a.rot)
+            {
+                #pragma unroll
+                for (int e2 = 0; e2 < 4; e2++)
+                {
+                    const int i0 = ks * 32 + 8 * g + 2 * e2;
+                    float x0 = 0.0f, x1 = 0.0f;
+                    if (i0 < a.rot)
+                    {
+                        x0 = bf16_to_f32(qr[i0]); x1 = bf16_to_f32(qr[i0 + 1]);
+                        if (i0 < a.rot_dims)
+                        {
+                            const float ang = (float)qpos * a.inv_freq[i0 >> 1];
+                            const float c = cosf(ang), sn = sinf(ang);
+                            const float u = x0, vv = x1;
+                            x0 = u * c - vv * sn; x1 = vv * c + u * sn;
+                        }
+                    }
+                    v[e2] = la_pack2(x0, x1);
+                }
+            }
+            qf[KSC + ks] = v;
+        }
+    }
+
+    f32x4 acc[NT];
+    #pragma unroll
+    for (int nt = 0; nt < NT; nt++) acc[nt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run[4], l_run[4];
+    #pragma unroll
+    for (int r = 0; r < 4; r++) { m_run[r] = -INFINITY; l_run[r] = 0.0f; }
+
+    const int k_lo = max(0, p0 - a.window + 1), k_hi = p0 + n - 1;
+    const int steps = (k_hi - k_lo + 1 + LA_KT - 1) / LA_KT;
+    const int per_split = (steps + a.nsplit - 1) / a.nsplit;
+    const int s_begin = split * per_split, s_end = min(steps, s_begin + per_split);
+    const int chunks_per_row = DP >> 3;
+
+    for (int st = s_begin; st < s_end; st++)
+    {
+        const int kbase = k_lo + st * LA_KT;
+        // stage 32 cache rows: row-major and (latent part) transposed
+        for (int c = t; c < LA_KT * chunks_per_row; c += 256)
+        {
+            const int key = c / chunks_per_row, ch = c - key * chunks_per_row;
+            const int j = min(kbase + key, k_hi);
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (ch * 8 < D) v = *(const u32x4*)(a.cache + ((long long)bt[j / a.page] * a.page + j % a.page) * D + ch * 8);
+            *(u32x4*)(Cs + key * CS + ch * 8) = v;
+            if (ch * 8 < R)
+            {
+                #pragma unroll
+                for (int e = 0; e < 4; e++)
+                {
+                    Ct[(ch * 8 + 2 * e) * LA_TS + key] = (u16)(v[e] & 0xffffu);
+                    Ct[(ch * 8 + 2 * e + 1) * LA_TS + key] = (u16)(v[e] >> 16);
+                }
+            }
+        }
+        block_sync();
+        float corr[4];
+        if (wave_live)
+        {
+            f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int ks = 0; ks < KSC; ks++)
+                if (ks * 32 < R)
+                {
+                    const u32x4 b0 = *(const u32x4*)(Cs + li * CS + ks * 32 + 8 * g);
+                    const u32x4 b1 = *(const u32x4*)(Cs + (16 + li) * CS + ks * 32 + 8 * g);
+                    s0 = mfma_16x16x32_bf16(qf[ks], b0, s0);
+                    s1 = mfma_16x16x32_bf16(qf[ks], b1, s1);
+                }
+            #pragma unroll
+            for (int ks = 0; ks < LA_ROT_STEPS; ks++)
+                if (ks * 32 < a.rot)
+                {
+                    const u32x4 b0 = *(const u32x4*)(Cs + li * CS + R + ks * 32 + 8 * g);
+                    const u32x4 b1 = *(const u32x4*)(Cs + (16 + li) * CS + R + ks * 32 + 8 * g);
+                    s0 = mfma_16x16x32_bf16(qf[KSC + ks], b0, s0);
+                    s1 = mfma_16x16x32_bf16(qf[KSC + ks], b1, s1);
+                }
+            #pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                const int qi = 4 * g + r;
+                const int qp = TR == 16 ? p0 + qi : p0;
+                const bool live_q = TR == 16 ? qi < n : true;
+                const int j0 = kbase + li, j1 = kbase + 16 + li;
+                const float v0 = live_q && j0 <= qp && j0 > qp - a.window ? s0[r] * a.scale : -INFINITY;
+                const float v1 = live_q && j1 <= qp && j1 > qp - a.window ? s1[r] * a.scale : -INFINITY;
+                const float mx = row16_allreduce_max(fmaxf(v0, v1));
+                const float m_new = fmaxf(m_run[r], mx);
+                const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+                const float e0 = expf(v0 - m_safe), e1 = expf(v1 - m_safe);
+                corr[r] = expf(m_run[r] - m_safe);
+                l_run[r] = l_run[r] * corr[r] + row16_allreduce_add(e0 + e1);
+                m_run[r] = m_new;
+                Ps[qi * LA_TS + li] = f32_to_bf16(e0);
+                Ps[qi * LA_TS + 16 + li] = f32_to_bf16(e1);
+            }
+        }
+        block_sync();
+        if (wave_live)
+        {
+            const u32x4 pa = *(const u32x4*)(Ps + li * LA_TS + 8 * g);
+            #pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                if (nt * 16 < R)
+                {
+                    f32x4 o = acc[nt];
+                    #pragma unroll
+                    for (int r = 0; r < 4; r++) o[r] *= corr[r];
+                    const u32x4 b = *(const u32x4*)(Ct + (nt * 16 + li) * LA_TS + 8 * g);
+                    acc[nt] = mfma_16x16x32_bf16(pa, b, o);
+                }
+        }
+        block_sync();
+    }
+    if (!wave_live) return;
+    #pragma unroll
+    for (int r = 0; r < 4; r++)
+    {
+        const int qi = 4 * g + r;
+        int orow, ohead;
+        if (TR == 16) { orow = r0 + qi; ohead = hb * 4 + w; if (qi >= n) continue; }
+        else { orow = r0; ohead = (hb * 4 + w) * 16 + qi; if (ohead >= H) continue; }
+        const long long vec = (long long)orow * H + ohead;
+        if (a.nsplit == 1)
+        {
+            const float inv = 1.0f / l_run[r];
+            #pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                if (nt * 16 < R) a.out[vec * R + nt * 16 + li] = f32_to_bf16(acc[nt][r] * inv);
+        }
+        else
+        {
+            float* po = a.part_o + (vec * a.nsplit + split) * R;
+            #pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                if (nt * 16 < R) po[nt * 16 + li] = acc[nt][r];
+            if (li == 0) { a.part_ml[(vec * a.nsplit + split) * 2] = m_run[r]; a.part_ml[(vec * a.nsplit + split) * 2 + 1] = l_run[r]; }
+        }
+    }
+}
+
+// joins the key splits of one query vector: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s
+KERNEL void __launch_bounds__(256) latent_attn_merge_kernel(const float* part_o, const float* part_ml, const int* vec_rows, int rows_h,
+                                                             int H, int R, int nsplit, u16* out)
+{
+    const int v = bid_x();                                   // index into the list of (row * H + head)
+    const long long vec = (long long)vec_rows[v / H] * H + v % H;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; s++) M = fmaxf(M, part_ml[(vec * nsplit + s) * 2]);
+    float L = 0.0f;
+    for (int s = 0; s < nsplit; s++)
+    {
+        const float m = part_ml[(vec * nsplit + s) * 2];
+        if (m != -INFINITY) L += expf(m - M) * part_ml[(vec * nsplit + s) * 2 + 1];
+    }
+    for (int i = tid(); i < R; i += 256)
+    {
+        float o = 0.0f;
+        for (int s = 0; s < nsplit; s++)
+        {
+            const float m = part_ml[(vec * nsplit + s) * 2];
+            if (m != -INFINITY) o = fmaf(expf(m - M), part_o[(vec * nsplit + s) * R + i], o);
+        }
+        out[vec * R + i] = f32_to_bf16(o / L);
+    }
+}
+
+template <int NT>
+static void launch_lat_mfma(const LatMfmaArgs& a, int tiles, int tile_rows, size_t smem, hipStream_t s)
+{
+    if (tile_rows == 16) LAUNCH((latent_attn_mfma_kernel<NT, 16>), dim3(tiles, (a.H + 3) / 4, a.nsplit), dim3(256), smem, s, a);
+    else LAUNCH((latent_attn_mfma_kernel<NT, 1>), dim3(tiles, (a.H + 63) / 64, a.nsplit), dim3(256), smem, s, a);
+}
+
 // ---- C ABI --------------------------------------------------------------------------------------------------------------------
 
 extern "C" int exl2_latent_append(const float* dkv, int ld, const void* norm_w, float eps, int dtype, int rows, int kv_rank, int rot,
@@ -207,6 +459,53 @@ extern "C" int exl2_latent_attn(const void* q, int ldq, int q_head_stride, int q
     const size_t smem = (size_t)(kv_rank + rot) * 4;
     if (dtype == 0) LAUNCH(latent_attn_kernel<u16>, dim3(rows, heads), dim3(256), smem, stream, a);
     else LAUNCH(latent_attn_kernel<float>, dim3(rows, heads), dim3(256), smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+/* the matrix-core form for bfloat16 (kv_rank a multiple of 32 and <= 512, rot a multiple of 8 and <= 128): the rows of the step are
+   given as tiles -- tile i covers rows tile_row0[i] .. + tile_rows[i] (<= 16 consecutive positions of ONE sequence) when
+   tile_mode is 16, or the single row tile_row0[i] when tile_mode is 1 (decoded tokens; all heads of the row share one pass over
+   the keys).  nsplit > 1 (tile_mode 1 only): the keys are split over workgroups, part_o fp32 [rows, heads, nsplit, kv_rank] and
+   part_ml fp32 [rows, heads, nsplit, 2] are scratch.  Returns EXL2_E_UNSUPPORTED for other shapes (use exl2_latent_attn). */
+extern "C" int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride, int q_rot_off, const float* q_abs, const void* cache,
+                                      int page, const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, void* out,
+                                      const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o, float* part_ml,
+                                      int nsplit, int heads, int kv_rank, int rot, int rot_dims, const float* inv_freq, float scale,
+                                      int window, void* stream)
+{
+    EXL2_REQUIRE(q && q_abs && cache && row_seq && row_pos && block_table && out && inv_freq && tile_row0, "latent_attn_tiles: null operand");
+    EXL2_REQUIRE(tile_mode == 16 || tile_mode == 1, "latent_attn_tiles: tile_mode is 16 or 1");
+    EXL2_REQUIRE(tile_mode == 1 || tile_rows, "latent_attn_tiles: tile_rows missing");
+    EXL2_REQUIRE(nsplit >= 1 && (nsplit == 1 || (tile_mode == 1 && part_o && part_ml)), "latent_attn_tiles: key splits need tile_mode 1 and scratch");
+    EXL2_REQUIRE(heads > 0 && page > 0 && window > 0 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent_attn_tiles: bad shape");
+    if (kv_rank % 32 != 0 || kv_rank > 512 || kv_rank <= 0 || rot % 8 != 0 || rot > 32 * LA_ROT_STEPS)
+        EXL2_FAIL(EXL2_E_UNSUPPORTED, "latent_attn_tiles: kv_rank %d / rot %d outside the matrix-core form", kv_rank, rot);
+    if (tiles <= 0) return EXL2_OK;
+    LatMfmaArgs a;
+    a.q = (const u16*)q; a.ldq = ldq; a.q_head_stride = q_head_stride; a.q_rot_off = q_rot_off; a.q_abs = q_abs;
+    a.cache = (const u16*)cache; a.page = page; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table; a.bt_stride = bt_stride;
+    a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.out = (u16*)out; a.part_o = part_o; a.part_ml = part_ml; a.nsplit = nsplit;
+    a.H = heads; a.R = kv_rank; a.rot = rot; a.rot_dims = rot_dims; a.inv_freq = inv_freq; a.scale = scale; a.window = window;
+    a.DP = (kv_rank + rot + 31) / 32 * 32;
+    const size_t smem = ((size_t)LA_KT * (a.DP + 8) + (size_t)kv_rank * LA_TS + 4 * 16 * LA_TS) * 2;
+    static bool attr_done[EXL2_MAX_DEVICES];
+    if (exl2_first_on_device(attr_done))
+    {
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<8, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<16, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<32, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<8, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<16, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<32, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (kv_rank <= 128) launch_lat_mfma<8>(a, tiles, tile_mode, smem, s);
+    else if (kv_rank <= 256) launch_lat_mfma<16>(a, tiles, tile_mode, smem, s);
+    else launch_lat_mfma<32>(a, tiles, tile_mode, smem, s);
+    if (nsplit > 1)
+        LAUNCH(latent_attn_merge_kernel, dim3(tiles * heads), dim3(256), 0, s, (const float*)part_o, (const float*)part_ml, tile_row0, tiles,
+               heads, kv_rank, nsplit, (u16*)out);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

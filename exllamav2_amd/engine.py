@@ -35,6 +35,7 @@ class Engine:
         of the entries and of `want`.  A request is admitted at its first entry.  `end`: requests whose pages and slot are given
         back after the step.  Returns fp32 logits [n wanted, vocab] on the device, or None."""
         ids, seq, pos, want_rows = [], [], [], []
+        t16_row0, t16_rows, t1_row0, t1_maxpos = [], [], [], 0
         seen = set()
         for rid, tokens, want in entries:
             if rid in seen:
@@ -48,6 +49,13 @@ class Engine:
             slot = self.slots[rid]
             start = self.pool.extend(slot, n)
             base = len(ids)
+            if n == 1:
+                t1_row0.append(base)
+                t1_maxpos = max(t1_maxpos, start)
+            else:
+                for i in range(0, n, 16):
+                    t16_row0.append(base + i)
+                    t16_rows.append(min(16, n - i))
             ids.extend(int(t) for t in tokens)
             seq.extend([slot] * n)
             pos.extend(range(start, start + n))
@@ -61,6 +69,11 @@ class Engine:
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
             batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows))
+            if t16_row0:
+                t16 = torch.tensor([t16_row0, t16_rows], dtype=torch.int32).to(dev)
+                batch.tiles16 = (t16[0], t16[1], len(t16_row0))
+            if t1_row0:
+                batch.tiles1 = (torch.tensor(t1_row0, dtype=torch.int32).to(dev), len(t1_row0), t1_maxpos)
             logits = self.model.step(batch, self.cache)
         for rid in end:
             self.finish(rid)

@@ -866,6 +866,23 @@ class ExtC:
                                                  int(kv_rank), int(rot), int(rot_dims), self._ptr(inv_freq, torch.float32, "inv_freq"),
                                                  float(scale), int(window), self._stream(out)))
 
+    @staticmethod
+    def latent_attn_tiles_supported(dtype, kv_rank: int, rot: int) -> bool:
+        """shapes of the matrix-core form of the latent attention (csrc/latent_attn.hip)"""
+        return dtype is torch.bfloat16 and kv_rank % 32 == 0 and 0 < kv_rank <= 512 and rot % 8 == 0 and rot <= 128
+
+    def latent_attn_tiles(self, q, ldq: int, q_head_stride: int, q_rot_off: int, q_abs, cache, page: int, row_seq, row_pos, block_table, out,
+                          tile_row0, tile_rows, tiles: int, tile_mode: int, heads: int, kv_rank: int, rot: int, rot_dims: int, inv_freq,
+                          scale: float, window: int, nsplit: int = 1, part_o=None, part_ml=None) -> None:
+        self.lib.check(self.lib.exl2_latent_attn_tiles(
+            self._ptr(q, torch.bfloat16, "q"), int(ldq), int(q_head_stride), int(q_rot_off), self._ptr(q_abs, torch.float32, "q_abs"),
+            self._ptr(cache, torch.bfloat16, "cache"), int(page), self._ptr(row_seq, torch.int32, "row_seq"),
+            self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1],
+            self._ptr(out, torch.bfloat16, "out"), self._ptr(tile_row0, torch.int32, "tile_row0"),
+            self._ptr(tile_rows, torch.int32, "tile_rows"), int(tiles), int(tile_mode), self._ptr(part_o, torch.float32, "part_o"),
+            self._ptr(part_ml, torch.float32, "part_ml"), int(nsplit), int(heads), int(kv_rank), int(rot), int(rot_dims),
+            self._ptr(inv_freq, torch.float32, "inv_freq"), float(scale), int(window), self._stream(out)))
+
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))
 

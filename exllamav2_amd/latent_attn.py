@@ -23,6 +23,8 @@ def rotary_inv_freq(base: float, dims: int, device) -> torch.Tensor:
 
 
 class LatentAttention:
+    KEYS_PER_SPLIT = 128                                  # decoded tokens: keys per workgroup of the split-key attention launch
+
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: int,
                  window: int, rot_base: float, rot_dims: int, scale: float, kv_from: int | None = None):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
@@ -84,8 +86,27 @@ class LatentAttention:
         q_abs = torch.empty((rows, H, R), dtype=torch.float32, device=dev)
         ext.dense_linear(q, self.uk_t.weight, q_abs, rows, R, dim, H * hs, dim, H * R, batch=H, sxb=hs, swb=R * dim, syb=R)
         o_lat = torch.empty((rows, H, R), dtype=dt, device=dev)
-        ext.latent_attn(q, H * hs, hs, dim, q_abs, rows_cache, pool.page_size, batch.row_seq, batch.row_pos, table, o_lat,
-                        rows, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window)
+        tiled = ext.latent_attn_tiles_supported(dt, R, rd) and (batch.tiles16 is not None or batch.tiles1 is not None)
+        if tiled:
+            # matrix-core kernels: portions of prompts as tiles of 16 positions x one head per wave, decoded tokens as one position x
+            # 16 heads per wave with the keys split over workgroups
+            common = (q, H * hs, hs, dim, q_abs, rows_cache, pool.page_size, batch.row_seq, batch.row_pos, table, o_lat)
+            if batch.tiles16 is not None:
+                row0, nrows, n = batch.tiles16
+                ext.latent_attn_tiles(*common, row0, nrows, n, 16, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window)
+            if batch.tiles1 is not None:
+                row0, n, max_pos = batch.tiles1
+                keys = min(self.window, max_pos + 1)
+                nsplit = max(1, min(32, -(-keys // self.KEYS_PER_SPLIT)))
+                part_o = part_ml = None
+                if nsplit > 1:
+                    part_o = torch.empty((rows, H, nsplit, R), dtype=torch.float32, device=dev)
+                    part_ml = torch.empty((rows, H, nsplit, 2), dtype=torch.float32, device=dev)
+                ext.latent_attn_tiles(*common, row0, None, n, 1, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window,
+                                      nsplit=nsplit, part_o=part_o, part_ml=part_ml)
+        else:
+            ext.latent_attn(q, H * hs, hs, dim, q_abs, rows_cache, pool.page_size, batch.row_seq, batch.row_pos, table, o_lat,
+                            rows, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window)
         og = torch.empty((rows, H * vd), dtype=dt, device=dev)
         ext.dense_linear(o_lat, self.uv.weight, og, rows, vd, R, H * R, R, H * vd, batch=H, sxb=R, swb=vd * R, syb=vd,
                          aux=f, ldaux=ncat, sauxb=vd, aux_off=self.off_g, epi=ext.EPI_MUL_SIGMOID_AUX)

@@ -54,6 +54,10 @@ class StepBatch:
     logit_rows: torch.Tensor
     rows: int
     n_logits: int
+    # rows grouped for tiled attention kernels: portions of prompts in tiles of <= 16 consecutive positions of one sequence
+    # (row0 int32 [n], rows int32 [n], n) and single decoded tokens (row0 int32 [n], n, largest position among them)
+    tiles16: tuple | None = None
+    tiles1: tuple | None = None
 
 
 class LayeredModel:

@@ -425,6 +425,16 @@ int exl2_latent_attn(const void* q, int ldq, int q_head_stride, int q_rot_off, c
                      const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, void* out, int dtype,
                      int rows, int heads, int kv_rank, int rot, int rot_dims, const float* inv_freq, float scale, int window,
                      void* stream);
+/* exl2_latent_attn on the matrix cores (bfloat16; kv_rank a multiple of 32 and <= 512, rot a multiple of 8 and <= 128; other shapes:
+   EXL2_E_UNSUPPORTED).  The step's rows come as tiles: tile i = rows tile_row0[i] .. + tile_rows[i] (<= 16 consecutive positions of
+   one sequence) with tile_mode 16, the single row tile_row0[i] with tile_mode 1 (a decoded token: its heads share one pass over
+   the keys).  nsplit > 1 (tile_mode 1): keys split over workgroups; part_o fp32 [rows, heads, nsplit, kv_rank] and part_ml fp32
+   [rows, heads, nsplit, 2] are scratch indexed by row. */
+int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride, int q_rot_off, const float* q_abs, const void* cache,
+                           int page, const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, void* out,
+                           const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o, float* part_ml,
+                           int nsplit, int heads, int kv_rank, int rot, int rot_dims, const float* inv_freq, float scale,
+                           int window, void* stream);
 
 #ifdef __cplusplus
 }

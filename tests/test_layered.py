@@ -176,14 +176,14 @@ def test_router_and_expert_mixture(be, experts, identity, top):
 # ---- the latent cache and its attention ----------------------------------------------------------------------------------------------
 
 
-def _attend_rows(be, dtype, R, rot, dims, H, window, page, n_tokens, dkv, q, q_abs, rows_at, base=100.0, scale=0.3):
+def _attend_rows(be, dtype, R, rot, dims, H, window, page, n_tokens, dkv, q, q_abs, rows_at, base=100.0, scale=0.3, tiles=None):
     """append n_tokens rows of one sequence (pages handed out in a scrambled order), then attend from the positions rows_at"""
     n_pages = -(-n_tokens // page) + 2
     order = list(range(n_pages))[::-1]
     table = np.zeros((2, n_pages), dtype=np.int32)
     table[1, :] = order
     cache = torch.zeros((n_pages, page, R + rot), dtype=dtype, device=be.device)
-    inv = be.t(np.array([base ** (-2.0 * i / dims) for i in range(max(1, dims // 2))], dtype=np.float32))
+    inv = be.t(np.array([base ** (-2.0 * i / max(dims, 1)) for i in range(max(1, dims // 2))], dtype=np.float32))
     seq = be.t(np.full(n_tokens, 1, dtype=np.int32))
     pos = be.t(np.arange(n_tokens, dtype=np.int32))
     nw = np.ones(R, dtype=np.float32)
@@ -191,8 +191,20 @@ def _attend_rows(be, dtype, R, rot, dims, H, window, page, n_tokens, dkv, q, q_a
     be.ext.latent_append(be.t(dkv), R + rot, dev(be, nw, dtype), 1e-6, n_tokens, R, rot, dims, inv, seq, pos, bt, page, cache)
     n = len(rows_at)
     out = torch.zeros((n, H, R), dtype=dtype, device=be.device)
-    be.ext.latent_attn(dev(be, q, dtype), H * rot, rot, 0, be.t(q_abs), cache, page, be.t(np.full(n, 1, dtype=np.int32)),
-                       be.t(np.array(rows_at, dtype=np.int32)), bt, out, n, H, R, rot, dims, inv, scale, window)
+    args = (dev(be, q, dtype), H * rot, rot, 0, be.t(q_abs), cache, page, be.t(np.full(n, 1, dtype=np.int32)),
+            be.t(np.array(rows_at, dtype=np.int32)), bt, out)
+    if tiles is None:
+        be.ext.latent_attn(*args, n, H, R, rot, dims, inv, scale, window)
+    elif tiles[0] == 16:                                         # rows_at are consecutive positions: tiles of <= 16 of them
+        row0 = list(range(0, n, 16))
+        be.ext.latent_attn_tiles(*args, be.t(np.array(row0, dtype=np.int32)), be.t(np.array([min(16, n - r) for r in row0], dtype=np.int32)),
+                                 len(row0), 16, H, R, rot, dims, inv, scale, window)
+    else:                                                        # every row a decoded token, keys split over tiles[1] workgroups
+        ns = tiles[1]
+        po = torch.zeros((n, H, ns, R), dtype=F32, device=be.device) if ns > 1 else None
+        pm = torch.zeros((n, H, ns, 2), dtype=F32, device=be.device) if ns > 1 else None
+        be.ext.latent_attn_tiles(*args, be.t(np.arange(n, dtype=np.int32)), None, n, 1, H, R, rot, dims, inv, scale, window,
+                                 nsplit=ns, part_o=po, part_ml=pm)
     return be.n(out.float())
 
 
@@ -223,14 +235,35 @@ def test_latent_attention_random(be, dtype, R, rot, dims, H, window, page):
     assert np.abs(got - want).max() <= (2e-5 if dtype is F32 else 3e-2)
 
 
+@pytest.mark.parametrize("R,rot,dims,H,window,page,n", [(32, 8, 8, 3, 5, 4, 40), (64, 16, 8, 5, 37, 8, 75), (160, 8, 8, 17, 1000, 16, 70),
+                                                         (32, 40, 40, 70, 33, 7, 50), (288, 8, 4, 2, 20, 16, 45)])
+@pytest.mark.parametrize("tiles", [(16, 1), (1, 1), (1, 3), (1, 8)])
+def test_latent_attention_on_the_matrix_cores(be, R, rot, dims, H, window, page, n, tiles):
+    """the bfloat16 tile kernels (portions: 16 positions x a head per wave; decoded tokens: a position x 16 heads per wave, keys split
+    over workgroups) against the plain restatement: head counts that do not fill a wave, windows that end inside a key step,
+    more splits than key steps, rotation over part of the rotated block"""
+    rng = np.random.default_rng(R + window + tiles[1])
+    dkv = bf16_exact(rng.standard_normal((n, R + rot)))
+    rows_at = list(range(n - 21, n)) if tiles[0] == 16 else [0, 1, min(window, n - 1), n - 1]
+    q = bf16_exact(rng.standard_normal((len(rows_at), H * rot)))
+    q_abs = bf16_exact(rng.standard_normal((len(rows_at), H, R)) * 0.5)
+    got = _attend_rows(be, BF16, R, rot, dims, H, window, page, n, dkv, q, q_abs, rows_at, tiles=tiles)
+    want = _attend_oracle(R, rot, dims, H, window, dkv, q, q_abs, rows_at)
+    assert np.abs(got - want).max() <= 3e-2
+
+
+@pytest.mark.parametrize("tiles", [None, (16, 1), (1, 1), (1, 4)])
 @pytest.mark.parametrize("many_rows", [False, True])
 @pytest.mark.parametrize("window,page,n,target_back", [(7, 4, 30, 6), (7, 4, 30, 7), (8, 8, 33, 7), (8, 8, 33, 8), (300, 16, 290, 289),
                                                         (300, 16, 290, 272), (5, 5, 6, 4), (5, 5, 6, 5)])
-def test_window_edge_stands_out(be, many_rows, window, page, n, target_back):
+def test_window_edge_stands_out(be, tiles, many_rows, window, page, n, target_back):
     """One key gets a score far above all others: `target_back` tokens behind the query.  Inside the window (target_back <
     window) the output IS that key's latent; one token outside it must not be seen at all.  Queries at the last position alone
     (a decoded token) or among many rows (a prompt's portion); targets at page borders, just inside / outside, and far back."""
-    R, rot, dims, H = 16, 4, 4, 2
+    R, rot, dims, H = (16, 4, 4, 2) if tiles is None else (32, 8, 8, 2)
+    if tiles is not None and (tiles[0] == 16) != many_rows:
+        pytest.skip("portions go to the 16-position tiles, single tokens to the one-position tiles")
+    dtype = F32 if tiles is None else BF16
     rng = np.random.default_rng(n + target_back)
     dkv = bf16_exact(rng.standard_normal((n, R + rot)))
     dkv[:, R:] = 0                                               # scores come from the latent part alone
@@ -240,12 +273,15 @@ def test_window_edge_stands_out(be, many_rows, window, page, n, target_back):
     rows_at = list(range(max(0, p - 9), n)) if many_rows else [p]
     q = np.zeros((len(rows_at), H * rot), dtype=np.float32)
     q_abs = (rng.standard_normal((len(rows_at), H, R)) * 0.05).astype(np.float32)
-    q_abs[-1, :, :] += (60.0 * c_t).astype(np.float32)           # score of the target ~ 60 |c|^2 * scale >> the rest
-    got = _attend_rows(be, F32, R, rot, dims, H, window, page, n, dkv, q, q_abs, rows_at)
+    boost = 60.0 if tiles is None else 8.0                       # (bfloat16 cache rows: a smaller boost keeps the OTHER scores' rounding small)
+    q_abs[-1, :, :] += (boost * c_t).astype(np.float32)          # score of the target ~ boost |c|^2 * scale >> the rest
+    if tiles is not None:
+        q_abs = bf16_exact(q_abs)
+    got = _attend_rows(be, dtype, R, rot, dims, H, window, page, n, dkv, q, q_abs, rows_at, tiles=tiles)
     want = _attend_oracle(R, rot, dims, H, window, dkv, q, q_abs, rows_at)
-    assert np.abs(got - want).max() <= 5e-5
+    assert np.abs(got - want).max() <= (5e-5 if tiles is None else 0.1)
     if target_back < window:
-        assert np.abs(got[-1] - c_t[None, :]).max() <= 1e-3
+        assert np.abs(got[-1] - c_t[None, :]).max() <= (1e-3 if tiles is None else 3e-2)
     else:
         assert np.abs(got[-1] - c_t[None, :]).max() > 0.2
 
