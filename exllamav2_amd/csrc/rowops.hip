@@ -181,29 +181,37 @@ KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const fl
     }
 }
 
-// per-expert row lists for the grouped linear: thread e scans all (token, choice) pairs in order (deterministic lists)
-KERNEL void __launch_bounds__(256) moe_group_kernel(const int* ids, int pairs, int n_real, int* count, int* offset, int* rows)
+// per-expert row lists for the grouped linear, in pair order.  Two launches of one workgroup per expert: counts (256 threads, ballot +
+// popcount), then offsets (sum of the counts in front) and an ordered compaction by one wave.
+KERNEL void __launch_bounds__(256) moe_count_kernel(const int* ids, int pairs, int* count)
 {
-    SHARED int cnt[256];
-    SHARED int off[256];
-    const int e = tid();
+    SHARED int part[4];
+    const int e = bid_x();
     int c = 0;
-    if (e < n_real)
-        for (int p = 0; p < pairs; p++) c += ids[p] == e;
-    cnt[e] = e < n_real ? c : 0;
-    block_sync();
-    if (e == 0)
+    for (int base = 0; base < pairs; base += 256)
     {
-        int run = 0;
-        for (int i = 0; i < n_real; i++) { off[i] = run; run += cnt[i]; }
+        const int p = base + tid();
+        c += __builtin_popcountll(wave_ballot(p < pairs && ids[p] == e));
     }
+    if (lane_id() == 0) part[wave_id()] = c;
     block_sync();
-    if (e < n_real)
+    if (tid() == 0) count[e] = part[0] + part[1] + part[2] + part[3];
+}
+
+KERNEL void __launch_bounds__(64) moe_fill_kernel(const int* ids, int pairs, const int* count, int* offset, int* rows)
+{
+    const int e = bid_x();
+    const int lane = lane_id();
+    int off = 0;
+    for (int i = 0; i < e; i++) off += count[i];
+    if (lane == 0) offset[e] = off;
+    for (int base = 0; base < pairs; base += 64)
     {
-        count[e] = cnt[e]; offset[e] = off[e];
-        int w = off[e];
-        for (int p = 0; p < pairs; p++)
-            if (ids[p] == e) rows[w++] = p;
+        const int p = base + lane;
+        const bool hit = p < pairs && ids[p] == e;
+        const u64 mask = wave_ballot(hit);
+        if (hit) rows[off + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = p;
+        off += __builtin_popcountll(mask);
     }
 }
 
@@ -274,8 +282,11 @@ extern "C" int exl2_moe_route_scored(const float* logits, const float* correctio
     if (grp_count)
     {
         EXL2_REQUIRE(grp_offset && grp_rows, "moe_route_scored: grouped lists need offsets and rows");
-        EXL2_REQUIRE(n_real <= 256, "moe_route_scored: grouped lists for at most 256 experts");
-        LAUNCH(moe_group_kernel, dim3(1), dim3(256), 0, stream, (const int*)ids, rows * top, n_real, grp_count, grp_offset, grp_rows);
+        if (n_real > 0)
+        {
+            LAUNCH(moe_count_kernel, dim3(n_real), dim3(256), 0, stream, (const int*)ids, rows * top, grp_count);
+            LAUNCH(moe_fill_kernel, dim3(n_real), dim3(64), 0, stream, (const int*)ids, rows * top, (const int*)grp_count, grp_offset, grp_rows);
+        }
     }
     HIP_TRY(hipGetLastError());
     return EXL2_OK;

@@ -16,13 +16,18 @@ from .layered import StepBatch
 
 
 class Engine:
-    def __init__(self, model, max_tokens: int, max_seqs: int = 4, page_size: int = PAGE_SIZE):
-        """The pool is made for `max_tokens` live tokens over at most `max_seqs` live requests, each holding whole pages."""
+    def __init__(self, model, max_tokens: int, max_seqs: int = 4, page_size: int = PAGE_SIZE, graphs: bool | None = None):
+        """The pool is made for `max_tokens` live tokens over at most `max_seqs` live requests, each holding whole pages.
+        graphs (default: on a GPU): steps that bring one token per request -- decoding -- replay ONE HIP graph per batch size; their
+        inputs (tokens, slots, positions, block table) live in device buffers the graph reads."""
         self.model = model
         pages = -(-int(max_tokens) // page_size) + max_seqs
         self.pool = PagePool(pages, page_size, max_seqs, model.device)
         self.cache = model.make_cache(self.pool)
         self.slots = {}                                           # request id -> slot
+        self.graphs = (model.device.type == "cuda") if graphs is None else bool(graphs)
+        self._decode = {}                                         # batch size -> captured decode step
+        self._stream = torch.cuda.Stream(device=model.device) if self.graphs and model.device.type == "cuda" else None
 
     def live(self):
         return list(self.slots)
@@ -64,7 +69,9 @@ class Engine:
                     raise RuntimeError(f"request {rid!r}: wanted place {w} outside its {n} tokens")
                 want_rows.append(base + w)
         logits = None
-        if ids:
+        if ids and self.graphs and not t16_row0 and len(want_rows) == len(ids):
+            logits = self._decode_step(ids, seq, pos)
+        elif ids:
             dev = self.model.device
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
@@ -75,9 +82,60 @@ class Engine:
             if t1_row0:
                 batch.tiles1 = (torch.tensor(t1_row0, dtype=torch.int32).to(dev), len(t1_row0), t1_maxpos)
             logits = self.model.step(batch, self.cache)
+            if logits is not None:
+                logits = logits.clone()                          # the step's own buffer is reused by the next step
         for rid in end:
             self.finish(rid)
         return logits
+
+    def _decode_step(self, ids, seq, pos):
+        """One token per request, every row's logits wanted: the step's launches are the same for every such step of this batch
+        size (the split of the attention keys is fixed by the pool's capacity), so they are captured once -- after a first eager
+        run that sizes the scratch arena -- and replayed with new inputs."""
+        m, ext, b = self.model, self.model.ext, len(ids)
+        st = self._decode.get(b)
+        if st is None:
+            dev = m.device
+            ar = torch.arange(b, dtype=torch.int32, device=dev)
+            st = {"inputs": torch.zeros((3, b), dtype=torch.int32, device=dev), "rows": ar, "graph": None, "runs": 0}
+            cap = self.pool.num_pages * self.pool.page_size
+            st["batch"] = StepBatch(st["inputs"][0], st["inputs"][1], st["inputs"][2], self.pool.device_table(), ar, b, b,
+                                    tiles1=(ar, b, cap - 1))
+            self._decode[b] = st
+        host = torch.tensor([ids, seq, pos], dtype=torch.int32)
+        if self._stream is None:                                   # (no GPU: the same batch, eagerly)
+            st["inputs"].copy_(host)
+            self.pool.device_table()
+            return m.step(st["batch"], self.cache).clone()
+        cur = torch.cuda.current_stream(m.device)
+        self._stream.wait_stream(cur)
+        with torch.cuda.stream(self._stream):
+            st["inputs"].copy_(host)
+            self.pool.device_table()
+            if st["graph"] is None:
+                logits = m.step(st["batch"], self.cache)          # eager: valid result, and every scratch buffer gets its size
+                st["runs"] += 1
+                if st["runs"] >= 2:                                # a batch size seen twice is worth a graph
+                    self._stream.synchronize()
+                    m.frozen = True
+                    ext.graph_begin_capture(self._stream.cuda_stream)
+                    try:
+                        st["logits"] = m.step(st["batch"], self.cache)    # recorded, not run
+                    finally:
+                        st["graph"] = ext.graph_end_capture(self._stream.cuda_stream)
+                        m.frozen = False
+            else:
+                ext.graph_launch(st["graph"], self._stream.cuda_stream)
+                logits = st["logits"]
+            out = logits.clone()
+        cur.wait_stream(self._stream)
+        return out
+
+    def close(self) -> None:
+        for st in self._decode.values():
+            if st.get("graph") is not None:
+                self.model.ext.graph_free(st["graph"])
+                st["graph"] = None
 
     def finish(self, rid) -> None:
         slot = self.slots.pop(rid, None)

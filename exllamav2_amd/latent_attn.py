@@ -72,10 +72,10 @@ class LatentAttention:
         H, dim, rd, vd, R = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         dt, dev = m.dtype, m.device
         ncat = self.front.out_features
-        f = self.front.forward(xh, rows, out_dtype=torch.float32)                       # [rows, dq | dkv | g] fp32
-        cq = torch.empty((rows, self.q_rank), dtype=dt, device=dev)
+        f = self.front.forward(xh, rows, out=m.buf("mix.f", (rows, ncat), torch.float32))     # [rows, dq | dkv | g] fp32
+        cq = m.buf("mix.cq", (rows, self.q_rank), dt)
         ext.rms_rows(f, ncat, self.dq_norm, False, cq, self.q_rank, rows, self.q_rank, m.norm_eps)
-        q = self.uq.forward(cq, rows)                                                    # [rows, H * (dim + rot)]
+        q = self.uq.forward(cq, rows, out=m.buf("mix.q", (rows, H * (dim + rd)), dt))
         pool = cache.pool
         rows_cache = cache.layer(self.layer_idx)
         table = batch.block_table
@@ -83,9 +83,9 @@ class LatentAttention:
             ext.latent_append(f, ncat, self.dkv_norm, m.norm_eps, rows, R, rd, self.rot_dims, self.inv_freq, batch.row_seq,
                               batch.row_pos, table, pool.page_size, rows_cache, dkv_off=self.off_dkv)
         hs = dim + rd
-        q_abs = torch.empty((rows, H, R), dtype=torch.float32, device=dev)
+        q_abs = m.buf("mix.q_abs", (rows, H, R), torch.float32)
         ext.dense_linear(q, self.uk_t.weight, q_abs, rows, R, dim, H * hs, dim, H * R, batch=H, sxb=hs, swb=R * dim, syb=R)
-        o_lat = torch.empty((rows, H, R), dtype=dt, device=dev)
+        o_lat = m.buf("mix.o_lat", (rows, H, R), dt)
         tiled = ext.latent_attn_tiles_supported(dt, R, rd) and (batch.tiles16 is not None or batch.tiles1 is not None)
         if tiled:
             # matrix-core kernels: portions of prompts as tiles of 16 positions x one head per wave, decoded tokens as one position x
@@ -100,14 +100,14 @@ class LatentAttention:
                 nsplit = max(1, min(32, -(-keys // self.KEYS_PER_SPLIT)))
                 part_o = part_ml = None
                 if nsplit > 1:
-                    part_o = torch.empty((rows, H, nsplit, R), dtype=torch.float32, device=dev)
-                    part_ml = torch.empty((rows, H, nsplit, 2), dtype=torch.float32, device=dev)
+                    part_o = m.buf("mix.part_o", (rows, H, nsplit, R), torch.float32)
+                    part_ml = m.buf("mix.part_ml", (rows, H, nsplit, 2), torch.float32)
                 ext.latent_attn_tiles(*common, row0, None, n, 1, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window,
                                       nsplit=nsplit, part_o=part_o, part_ml=part_ml)
         else:
             ext.latent_attn(q, H * hs, hs, dim, q_abs, rows_cache, pool.page_size, batch.row_seq, batch.row_pos, table, o_lat,
                             rows, H, R, rd, self.rot_dims, self.inv_freq, self.scale, self.window)
-        og = torch.empty((rows, H * vd), dtype=dt, device=dev)
+        og = m.buf("mix.og", (rows, H * vd), dt)
         ext.dense_linear(o_lat, self.uv.weight, og, rows, vd, R, H * R, R, H * vd, batch=H, sxb=R, swb=vd * R, syb=vd,
                          aux=f, ldaux=ncat, sauxb=vd, aux_off=self.off_g, epi=ext.EPI_MUL_SIGMOID_AUX)
-        return self.o.forward(og, rows, out_dtype=torch.float32)
+        return self.o.forward(og, rows, out=m.buf("mix.y", (rows, m.width), torch.float32))

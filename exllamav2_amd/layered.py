@@ -68,6 +68,23 @@ class LayeredModel:
         self.width, self.vocab, self.norm_eps = config.width, config.vocab, config.norm_eps
         self.layers = []
         self.loaded = False
+        self._scratch = {}
+        self.frozen = False                               # True while a step is being captured into a graph: scratch may not grow
+
+    def buf(self, tag: str, shape, dtype) -> torch.Tensor:
+        """A view of the model's scratch arena: one persistent buffer per tag (grown on demand), so the addresses a step uses stay
+        the same from step to step -- what a captured graph needs -- and nothing is allocated on the hot path.  Tags are unique
+        among the buffers that are alive at the same time; layers run one after the other and share them."""
+        n = 1
+        for d in shape:
+            n *= int(d)
+        t = self._scratch.get(tag)
+        if t is None or t.dtype is not dtype or t.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"scratch buffer '{tag}' would have to grow while a step is being captured")
+            t = torch.empty((max(n, 1),), dtype=dtype, device=self.device)
+            self._scratch[tag] = t
+        return t[:n].view(*shape)
 
     # ---- loading --------------------------------------------------------------------------------------------------------------
 
@@ -137,21 +154,21 @@ class LayeredModel:
         """Runs the batch's rows through all layers, appending to the cache; returns fp32 logits [n_logits, vocab] (None if
         no row wants them)."""
         ext, cfg, rows = self.ext, self.config, batch.rows
-        x32 = torch.empty((rows, self.width), dtype=torch.float32, device=self.device)
-        xh = x32 if self.dtype is torch.float32 else torch.empty((rows, self.width), dtype=self.dtype, device=self.device)
+        x32 = self.buf("x32", (rows, self.width), torch.float32)
+        xh = x32 if self.dtype is torch.float32 else self.buf("xh", (rows, self.width), self.dtype)
         ext.embed_scale(self.embed, batch.ids, x32, xh, cfg.embedding_scale)
         for mixer, norm1, ff, norm2 in self.layers:
             y = mixer.forward(xh, rows, batch, cache)
             norm1.forward(x32, xh, y, rows)
             if norm2 is not None:
                 if ff is None:
-                    y, mix = torch.zeros_like(x32), None
+                    y, mix = self.buf("zero", (rows, self.width), torch.float32).zero_(), None
                 else:
                     y, mix = ff.forward(xh, rows)
                 norm2.forward(x32, xh, y, rows, moe=mix)
         if batch.n_logits == 0:
             return None
-        xn = torch.empty((batch.n_logits, self.width), dtype=self.dtype, device=self.device)
+        xn = self.buf("xn", (batch.n_logits, self.width), self.dtype)
         ext.rms_rows(x32, self.width, self.final_norm, True, xn, self.width, batch.n_logits, self.width, cfg.norm_eps,
                      row_idx=batch.logit_rows)
-        return self.head.forward(xn, batch.n_logits, out_dtype=torch.float32)
+        return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), torch.float32))

@@ -60,6 +60,7 @@ class DenseGatedMLP:
         return self.gate.weight_bytes() + self.up.weight_bytes() + self.down.weight_bytes()
 
     def forward(self, xh: torch.Tensor, rows: int):
-        g = self.gate.forward(xh, rows, out_dtype=torch.float32)
-        a = self.up.forward(xh, rows, aux=g, aux_ld=g.shape[-1], epi=self.ext.EPI_SILU_AUX_MUL)
-        return self.down.forward(a, rows, out_dtype=torch.float32), None
+        m, ff = self.model, self.gate.out_features
+        g = self.gate.forward(xh, rows, out=m.buf("ff.g", (rows, ff), torch.float32))
+        a = self.up.forward(xh, rows, out=m.buf("ff.a", (rows, ff), m.dtype), aux=g, aux_ld=ff, epi=self.ext.EPI_SILU_AUX_MUL)
+        return self.down.forward(a, rows, out=m.buf("ff.y", (rows, m.width), torch.float32)), None

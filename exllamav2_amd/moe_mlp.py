@@ -96,21 +96,20 @@ class ScoredMoEMLP:
         E, top, ff, width = self.experts, self.top, self.ff, m.width
         dev, dt = m.device, m.dtype
         n_total = E + self.identity
-        logits = self.router.forward(xh, rows, out_dtype=torch.float32)
-        ids = torch.empty((rows, top), dtype=torch.int32, device=dev)
-        wts = torch.empty((rows, top), dtype=torch.float32, device=dev)
+        logits = self.router.forward(xh, rows, out=m.buf("moe.logits", (rows, n_total), torch.float32))
+        ids = m.buf("moe.ids", (rows, top), torch.int32)
+        wts = m.buf("moe.wts", (rows, top), torch.float32)
         pairs = rows * top
         grouped = pairs > self.PAIR_ROWS_MAX and E > 0
         groups = None
         if grouped:
-            groups = (torch.empty((E,), dtype=torch.int32, device=dev), torch.empty((E,), dtype=torch.int32, device=dev),
-                      torch.empty((pairs,), dtype=torch.int32, device=dev))
+            groups = (m.buf("moe.count", (E,), torch.int32), m.buf("moe.offset", (E,), torch.int32), m.buf("moe.rows", (pairs,), torch.int32))
         ext.moe_route_scored(logits, self.correction, ids, wts, rows, n_total, top, self.route_scale, E, groups=groups)
         if E == 0:
             return None, (None, ids, wts, 0)
-        g = torch.empty((pairs, ff), dtype=torch.float32, device=dev)
-        a = torch.empty((pairs, ff), dtype=dt, device=dev)
-        y = torch.empty((pairs, width), dtype=torch.float32, device=dev)
+        g = m.buf("ff.g", (pairs, ff), torch.float32)
+        a = m.buf("ff.a", (pairs, ff), dt)
+        y = m.buf("ff.y", (pairs, width), torch.float32)
         if grouped:
             kw = dict(batch=E, groups=groups)
         else:
