@@ -1,11 +1,12 @@
 // dense.hip -- linears over UNQUANTIZED weights (bfloat16 or fp32, stored [out, in]) for gfx950, + their C ABI.
 //
-// y[r, n] = epilogue( sum_k x[r, k] * w[n, k] ), fp32 accumulation always.  One entry point, three kernels:
+// y[r, n] = epilogue( sum_k x[r, k] * w[n, k] ), fp32 accumulation always.  One entry point, four kernels:
 //   * lin_rows_kernel  -- decode-sized calls (<= 16 rows): one wave per output column, the K range split over the 64 lanes with
 //                         16-byte loads of the weight row (a [out, in] row is contiguous: one wave streams it once for all rows);
 //                         also the sparse-MoE decode form: every row names the weight slab it multiplies (w_sel).
-//   * lin_mfma_kernel  -- bfloat16, many rows: v_mfma_f32_16x16x32_bf16.  Both operands are K-contiguous, so a lane's 8 values of an
-//                         A or B fragment are ONE 16-byte load straight from memory into the register the matrix core reads.
+//   * lin_mfma_kernel  -- bfloat16, 17 .. 64 rows: v_mfma_f32_16x16x32_bf16.  Both operands are K-contiguous, so a lane's 8 values of
+//                         an A or B fragment are ONE 16-byte load straight from memory into the register the matrix core reads.
+//   * lin_mfma_tile_kernel -- bfloat16, more rows: 128 x 128 tiles staged through LDS, two stages deep.
 //   * lin_tile_kernel  -- fp32 (true 32-bit FMA, no reduced-precision matrix mode) and every shape the other two decline
 //                         (K or a leading dimension that is not a multiple of 8 values): 64 x 64 tiles through LDS.
 // A call may be batched over blockIdx.z (per-head projections: element offsets per batch for x, w, y, aux) or GROUPED (sparse MoE
@@ -284,6 +285,103 @@ KERNEL void __launch_bounds__(256) lin_mfma_kernel(const LinArgs a)
         }
 }
 
+// ---- bfloat16 on the matrix cores, 128 x 128 tiles through LDS (many rows) ------------------------------------------------------
+// Workgroup = 4 waves = 128 rows x 128 columns, a wave owns a 64 x 64 quadrant (4 x 4 fragments).  A K step is 32 values: the
+// workgroup stages the 128 x 32 slices of x and w (16 bytes per thread and row, row stride 80 bytes: the 16-lane phases of a
+// 16-byte LDS read fall into distinct banks), two stages deep -- the next step's slices are requested from memory before the current
+// step's 16 MFMAs and written to the other stage after them.
+
+#define LT_STRIDE 40                                         // values per staged row (32 + 8 of padding)
+
+template <typename TY>
+KERNEL void __launch_bounds__(256) lin_mfma_tile_kernel(const LinArgs a)
+{
+    SHARED __attribute__((aligned(16))) u16 As[2][128 * LT_STRIDE];
+    SHARED __attribute__((aligned(16))) u16 Bs[2][128 * LT_STRIDE];
+    SHARED int rowmap[128];
+    const int z = bid_z();
+    const int m0 = bid_y() * 128, n0 = bid_x() * 128;
+    const int M = a.grp_count ? a.grp_count[z] : a.M;
+    if (m0 >= M) return;
+    const int t = tid(), lane = lane_id(), w = wave_id();
+    if (t < 128)
+    {
+        const int r = min(m0 + t, M - 1);
+        rowmap[t] = a.grp_rows ? a.grp_rows[a.grp_offset[z] + r] : r;
+    }
+    block_sync();
+    // staging: thread t brings chunk (t & 3) of rows (t >> 2) and (t >> 2) + 64 of both slices
+    const int sr = t >> 2, sc = (t & 3) * 8;
+    const u16* xp0 = (const u16*)a.x + (long long)z * a.sxb + (long long)(rowmap[sr] / a.x_div) * a.ldx + sc;
+    const u16* xp1 = (const u16*)a.x + (long long)z * a.sxb + (long long)(rowmap[sr + 64] / a.x_div) * a.ldx + sc;
+    const u16* wp0 = (const u16*)a.w + (long long)z * a.swb + (long long)min(n0 + sr, a.N - 1) * a.ldw + sc;
+    const u16* wp1 = (const u16*)a.w + (long long)z * a.swb + (long long)min(n0 + sr + 64, a.N - 1) * a.ldw + sc;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const int li = lane & 15, kg = (lane >> 4) * 8;
+    const int wm = (w >> 1) * 64, wn = (w & 1) * 64;
+    f32x4 acc[4][4];
+    #pragma unroll
+    for (int i = 0; i < 4; i++)
+        #pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4 ra0, ra1, rb0, rb1;
+    {
+        const bool live = sc < a.K;
+        ra0 = live ? *(const u32x4*)xp0 : zero; ra1 = live ? *(const u32x4*)xp1 : zero;
+        rb0 = live ? *(const u32x4*)wp0 : zero; rb1 = live ? *(const u32x4*)wp1 : zero;
+    }
+    *(u32x4*)&As[0][sr * LT_STRIDE + sc] = ra0; *(u32x4*)&As[0][(sr + 64) * LT_STRIDE + sc] = ra1;
+    *(u32x4*)&Bs[0][sr * LT_STRIDE + sc] = rb0; *(u32x4*)&Bs[0][(sr + 64) * LT_STRIDE + sc] = rb1;
+    block_sync();
+    int stage = 0;
+    for (int k0 = 0; k0 < a.K; k0 += 32)
+    {
+        const int kn = k0 + 32;
+        if (kn < a.K)
+        {
+            const bool live = kn + sc < a.K;
+            ra0 = live ? *(const u32x4*)(xp0 + kn) : zero; ra1 = live ? *(const u32x4*)(xp1 + kn) : zero;
+            rb0 = live ? *(const u32x4*)(wp0 + kn) : zero; rb1 = live ? *(const u32x4*)(wp1 + kn) : zero;
+        }
+        u32x4 af[4], bf[4];
+        #pragma unroll
+        for (int i = 0; i < 4; i++) af[i] = *(const u32x4*)&As[stage][(wm + 16 * i + li) * LT_STRIDE + kg];
+        #pragma unroll
+        for (int j = 0; j < 4; j++) bf[j] = *(const u32x4*)&Bs[stage][(wn + 16 * j + li) * LT_STRIDE + kg];
+        #pragma unroll
+        for (int i = 0; i < 4; i++)
+            #pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = mfma_16x16x32_bf16(af[i], bf[j], acc[i][j]);
+        if (kn < a.K)
+        {
+            const int o = stage ^ 1;
+            *(u32x4*)&As[o][sr * LT_STRIDE + sc] = ra0; *(u32x4*)&As[o][(sr + 64) * LT_STRIDE + sc] = ra1;
+            *(u32x4*)&Bs[o][sr * LT_STRIDE + sc] = rb0; *(u32x4*)&Bs[o][(sr + 64) * LT_STRIDE + sc] = rb1;
+        }
+        block_sync();
+        stage ^= 1;
+    }
+    #pragma unroll
+    for (int i = 0; i < 4; i++)
+        #pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int rl = wm + 16 * i + 4 * (lane >> 4) + r;
+            if (m0 + rl >= M) continue;
+            const long long row = rowmap[rl];
+            #pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                const int n = n0 + wn + 16 * j + li;
+                if (n >= a.N) continue;
+                float aux = 0.0f;
+                if (a.epi != EPI_NONE) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
+                st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r], aux, a.limit));
+            }
+        }
+}
+
 // ---- host -------------------------------------------------------------------------------------------------------------------
 
 template <typename T, typename TY, bool VEC>
@@ -309,7 +407,8 @@ static void launch_dense(const LinArgs& a, int batch, bool vec_ok, int max_rows,
         if (vec_ok)
         {
             if (max_rows <= 32) LAUNCH((lin_mfma_kernel<TY, 2>), dim3((a.N + 255) / 256, (max_rows + 31) / 32, batch), dim3(256), 0, s, a);
-            else LAUNCH((lin_mfma_kernel<TY, 4>), dim3((a.N + 255) / 256, (max_rows + 63) / 64, batch), dim3(256), 0, s, a);
+            else if (max_rows <= 64) LAUNCH((lin_mfma_kernel<TY, 4>), dim3((a.N + 255) / 256, (max_rows + 63) / 64, batch), dim3(256), 0, s, a);
+            else LAUNCH((lin_mfma_tile_kernel<TY>), dim3((a.N + 127) / 128, (max_rows + 127) / 128, batch), dim3(256), 0, s, a);
             return;
         }
     }

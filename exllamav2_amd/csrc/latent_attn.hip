@@ -284,9 +284,11 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     {
         const int kbase = k_lo + st * LA_KT;
         // stage 32 cache rows: row-major and (latent part) transposed
+        // (consecutive threads take consecutive KEYS of one 16-byte chunk: the transposed 2-byte stores of a wave then fall into
+        // consecutive LDS addresses instead of one bank)
         for (int c = t; c < LA_KT * chunks_per_row; c += 256)
         {
-            const int key = c / chunks_per_row, ch = c - key * chunks_per_row;
+            const int key = c & (LA_KT - 1), ch = c >> 5;
             const int j = min(kbase + key, k_hi);
             u32x4 v = {0u, 0u, 0u, 0u};
             if (ch * 8 < D) v = *(const u32x4*)(a.cache + ((long long)bt[j / a.page] * a.page + j % a.page) * D + ch * 8);

@@ -42,7 +42,8 @@ TOL = {F32: 3e-5, BF16: 4e-2}
 
 @pytest.mark.parametrize("dtype,M,N,K", [(F32, 1, 9, 40), (F32, 5, 70, 36), (F32, 13, 8, 21), (F32, 33, 66, 50), (F32, 70, 10, 8),
                                          (BF16, 1, 12, 64), (BF16, 3, 7, 24), (BF16, 16, 33, 40), (BF16, 17, 40, 64), (BF16, 45, 300, 72),
-                                         (BF16, 100, 20, 8), (BF16, 21, 19, 20), (BF16, 4, 6, 10)])
+                                         (BF16, 100, 20, 8), (BF16, 21, 19, 20), (BF16, 4, 6, 10), (BF16, 130, 150, 72), (BF16, 70, 130, 200),
+                                         (BF16, 260, 24, 40)])
 @pytest.mark.parametrize("epi", [0, 1, 2, 3])
 def test_dense_linear(be, dtype, M, N, K, epi):
     rng = np.random.default_rng(M * 1000 + N * 10 + K + epi)
