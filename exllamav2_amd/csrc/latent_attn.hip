@@ -197,6 +197,7 @@ struct LatMfmaArgs
 #define LA_KT 32
 #define LA_TS 40                                             // row stride (values) of the transposed and the probability tiles
 #define LA_ROT_STEPS 4
+#define LA_STAGE_IT 10                                       // 16-byte chunks per thread and key step: (512 + 128) / 8 / 8
 
 DEV u32 la_pack2(float lo, float hi) { return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16); }
 
@@ -279,31 +280,61 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     const int per_split = (steps + a.nsplit - 1) / a.nsplit;
     const int s_begin = split * per_split, s_end = min(steps, s_begin + per_split);
     const int chunks_per_row = DP >> 3;
-
-    for (int st = s_begin; st < s_end; st++)
-    {
-        const int kbase = k_lo + st * LA_KT;
-        // stage 32 cache rows: row-major and (latent part) transposed
-        // (consecutive threads take consecutive KEYS of one 16-byte chunk: the transposed 2-byte stores of a wave then fall into
-        // consecutive LDS addresses instead of one bank)
-        for (int c = t; c < LA_KT * chunks_per_row; c += 256)
+    // Staging, software-pipelined: thread t always brings key (t & 31) of a step -- chunks (t >> 5) + 8 i of that cache row -- so one
+    // block-table lookup per thread and step names the row, and the row's 16-byte loads are independent of each other.  The loads
+    // of step s + 1 are issued before the matrix products of step s and land in registers meanwhile; the row of step s + 2 is
+    // looked up behind them.  (Consecutive threads = consecutive keys: the transposed 2-byte LDS stores of a wave are contiguous.)
+    const int skey = t & (LA_KT - 1), sch0 = t >> 5;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    u32x4 sv[LA_STAGE_IT];
+    auto key_row = [&](int st) -> long long {
+        const int j = min(k_lo + st * LA_KT + skey, k_hi);
+        return ((long long)bt[j / a.page] * a.page + j % a.page) * D;
+    };
+    auto issue = [&](long long rowoff) {
+        #pragma unroll
+        for (int it = 0; it < LA_STAGE_IT; it++)
         {
-            const int key = c & (LA_KT - 1), ch = c >> 5;
-            const int j = min(kbase + key, k_hi);
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (ch * 8 < D) v = *(const u32x4*)(a.cache + ((long long)bt[j / a.page] * a.page + j % a.page) * D + ch * 8);
-            *(u32x4*)(Cs + key * CS + ch * 8) = v;
+            const int ch = sch0 + 8 * it;
+            sv[it] = ch * 8 < D ? *(const u32x4*)(a.cache + rowoff + ch * 8) : zero4;
+        }
+    };
+    auto commit = [&]() {
+        #pragma unroll
+        for (int it = 0; it < LA_STAGE_IT; it++)
+        {
+            const int ch = sch0 + 8 * it;
+            if (ch >= chunks_per_row) continue;
+            const u32x4 v = sv[it];
+            *(u32x4*)(Cs + skey * CS + ch * 8) = v;
             if (ch * 8 < R)
             {
                 #pragma unroll
                 for (int e = 0; e < 4; e++)
                 {
-                    Ct[(ch * 8 + 2 * e) * LA_TS + key] = (u16)(v[e] & 0xffffu);
-                    Ct[(ch * 8 + 2 * e + 1) * LA_TS + key] = (u16)(v[e] >> 16);
+                    Ct[(ch * 8 + 2 * e) * LA_TS + skey] = (u16)(v[e] & 0xffffu);
+                    Ct[(ch * 8 + 2 * e + 1) * LA_TS + skey] = (u16)(v[e] >> 16);
                 }
             }
         }
+    };
+    long long row_next = 0;
+    if (s_begin < s_end)
+    {
+        issue(key_row(s_begin));
+        if (s_begin + 1 < s_end) row_next = key_row(s_begin + 1);
+    }
+
+    for (int st = s_begin; st < s_end; st++)
+    {
+        const int kbase = k_lo + st * LA_KT;
+        commit();
         block_sync();
+        if (st + 1 < s_end)
+        {
+            issue(row_next);
+            if (st + 2 < s_end) row_next = key_row(st + 2);
+        }
         float corr[4];
         if (wave_live)
         {
