@@ -197,11 +197,15 @@ struct LatMfmaArgs
 #define LA_KT 32
 #define LA_TS 40                                             // row stride (values) of the transposed and the probability tiles
 #define LA_ROT_STEPS 4
+#define LA_MAX_SPLIT 32
 #define LA_STAGE_IT 10                                       // 16-byte chunks per thread and key step: (512 + 128) / 8 / 8
 
 DEV u32 la_pack2(float lo, float hi) { return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16); }
 
-template <int NT, int TR>
+// RS > 0: the EXACT form -- kv_rank == 16 NT and rot == 32 RS are compile-time constants, so every size guard below folds away and the
+// unrolled loops become straight-line code the scheduler can reorder (LDS reads of the next fragments ahead of the current matrix
+// products).  RS == 0: sizes from the arguments (any kv_rank % 32 == 0, rot % 8 == 0).
+template <int NT, int TR, int RS>
 KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
 {
     DYN_SMEM(smem);
@@ -211,7 +215,9 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     const int n = TR == 16 ? a.tile_rows[tile] : 1;
     const int p0 = a.row_pos[r0];
     const int* bt = a.block_table + (long long)a.row_seq[r0] * a.bt_stride;
-    const int H = a.H, R = a.R, D = a.R + a.rot, DP = a.DP, CS = DP + 8;
+    const int H = a.H;
+    const int R = RS > 0 ? NT * 16 : a.R, rot = RS > 0 ? RS * 32 : a.rot;
+    const int D = R + rot, DP = RS > 0 ? D : a.DP, CS = DP + 8;
     u16* Cs = (u16*)smem;                                    // [32][CS]
     u16* Ct = Cs + LA_KT * CS;                               // [R][LA_TS]
     u16* Ps = Ct + R * LA_TS + w * 16 * LA_TS;               // [16][LA_TS], this wave's
@@ -243,14 +249,14 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
         for (int ks = 0; ks < LA_ROT_STEPS; ks++)
         {
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (ks * 32 < a.rot)
+            if (ks * 32 < rot)
             {
                 #pragma unroll
                 for (int e2 = 0; e2 < 4; e2++)
                 {
                     const int i0 = ks * 32 + 8 * g + 2 * e2;
                     float x0 = 0.0f, x1 = 0.0f;
-                    if (i0 < a.rot)
+                    if (i0 < rot)
                     {
                         x0 = bf16_to_f32(qr[i0]); x1 = bf16_to_f32(qr[i0 + 1]);
                         if (i0 < a.rot_dims)
@@ -329,7 +335,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     {
         const int kbase = k_lo + st * LA_KT;
         commit();
-        block_sync();
+        block_sync_lds();                                 // (LDS-only barriers: the loads issued below stay in flight across them)
         if (st + 1 < s_end)
         {
             issue(row_next);
@@ -350,7 +356,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                 }
             #pragma unroll
             for (int ks = 0; ks < LA_ROT_STEPS; ks++)
-                if (ks * 32 < a.rot)
+                if (ks * 32 < rot)
                 {
                     const u32x4 b0 = *(const u32x4*)(Cs + li * CS + R + ks * 32 + 8 * g);
                     const u32x4 b1 = *(const u32x4*)(Cs + (16 + li) * CS + R + ks * 32 + 8 * g);
@@ -377,7 +383,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                 Ps[qi * LA_TS + 16 + li] = f32_to_bf16(e1);
             }
         }
-        block_sync();
+        block_sync_lds();
         if (wave_live)
         {
             const u32x4 pa = *(const u32x4*)(Ps + li * LA_TS + 8 * g);
@@ -392,7 +398,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                     acc[nt] = mfma_16x16x32_bf16(pa, b, o);
                 }
         }
-        block_sync();
+        block_sync_lds();
     }
     if (!wave_live) return;
     #pragma unroll
@@ -427,31 +433,58 @@ KERNEL void __launch_bounds__(256) latent_attn_merge_kernel(const float* part_o,
 {
     const int v = bid_x();                                   // index into the list of (row * H + head)
     const long long vec = (long long)vec_rows[v / H] * H + v % H;
+    // (all loads first, unconditionally: a load under a branch is a round trip of its own)
+    float ms[LA_MAX_SPLIT], wt[LA_MAX_SPLIT];
     float M = -INFINITY;
-    for (int s = 0; s < nsplit; s++) M = fmaxf(M, part_ml[(vec * nsplit + s) * 2]);
+    #pragma unroll
+    for (int s = 0; s < LA_MAX_SPLIT; s++) { ms[s] = part_ml[(vec * nsplit + min(s, nsplit - 1)) * 2]; wt[s] = part_ml[(vec * nsplit + min(s, nsplit - 1)) * 2 + 1]; }
+    #pragma unroll
+    for (int s = 0; s < LA_MAX_SPLIT; s++) if (s < nsplit) M = fmaxf(M, ms[s]);
     float L = 0.0f;
-    for (int s = 0; s < nsplit; s++)
+    #pragma unroll
+    for (int s = 0; s < LA_MAX_SPLIT; s++)
     {
-        const float m = part_ml[(vec * nsplit + s) * 2];
-        if (m != -INFINITY) L += expf(m - M) * part_ml[(vec * nsplit + s) * 2 + 1];
+        const float e = s < nsplit && ms[s] != -INFINITY ? expf(ms[s] - M) : 0.0f;
+        L = fmaf(e, wt[s], L);
+        wt[s] = e;
     }
     for (int i = tid(); i < R; i += 256)
     {
+        float pv[LA_MAX_SPLIT];
+        #pragma unroll
+        for (int s = 0; s < LA_MAX_SPLIT; s++) pv[s] = part_o[(vec * nsplit + min(s, nsplit - 1)) * R + i];
         float o = 0.0f;
-        for (int s = 0; s < nsplit; s++)
-        {
-            const float m = part_ml[(vec * nsplit + s) * 2];
-            if (m != -INFINITY) o = fmaf(expf(m - M), part_o[(vec * nsplit + s) * R + i], o);
-        }
+        #pragma unroll
+        for (int s = 0; s < LA_MAX_SPLIT; s++) o = fmaf(wt[s], s < nsplit ? pv[s] : 0.0f, o);
         out[vec * R + i] = f32_to_bf16(o / L);
     }
+}
+
+template <int NT, int TR, int RS>
+static void launch_lat_mfma_one(const LatMfmaArgs& a, int tiles, size_t smem, hipStream_t s)
+{
+    static bool attr_done[EXL2_MAX_DEVICES];
+    if (exl2_first_on_device(attr_done))
+        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<NT, TR, RS>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    LAUNCH((latent_attn_mfma_kernel<NT, TR, RS>), dim3(tiles, TR == 16 ? (a.H + 3) / 4 : (a.H + 63) / 64, a.nsplit), dim3(256), smem, s, a);
 }
 
 template <int NT>
 static void launch_lat_mfma(const LatMfmaArgs& a, int tiles, int tile_rows, size_t smem, hipStream_t s)
 {
-    if (tile_rows == 16) LAUNCH((latent_attn_mfma_kernel<NT, 16>), dim3(tiles, (a.H + 3) / 4, a.nsplit), dim3(256), smem, s, a);
-    else LAUNCH((latent_attn_mfma_kernel<NT, 1>), dim3(tiles, (a.H + 63) / 64, a.nsplit), dim3(256), smem, s, a);
+    const int rs = a.R == NT * 16 && (a.rot == 32 || a.rot == 64) ? a.rot / 32 : 0;
+    if (tile_rows == 16)
+    {
+        if (rs == 1) launch_lat_mfma_one<NT, 16, 1>(a, tiles, smem, s);
+        else if (rs == 2) launch_lat_mfma_one<NT, 16, 2>(a, tiles, smem, s);
+        else launch_lat_mfma_one<NT, 16, 0>(a, tiles, smem, s);
+    }
+    else
+    {
+        if (rs == 1) launch_lat_mfma_one<NT, 1, 1>(a, tiles, smem, s);
+        else if (rs == 2) launch_lat_mfma_one<NT, 1, 2>(a, tiles, smem, s);
+        else launch_lat_mfma_one<NT, 1, 0>(a, tiles, smem, s);
+    }
 }
 
 // ---- C ABI --------------------------------------------------------------------------------------------------------------------
@@ -510,6 +543,7 @@ extern "C" int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride,
     EXL2_REQUIRE(q && q_abs && cache && row_seq && row_pos && block_table && out && inv_freq && tile_row0, "latent_attn_tiles: null operand");
     EXL2_REQUIRE(tile_mode == 16 || tile_mode == 1, "latent_attn_tiles: tile_mode is 16 or 1");
     EXL2_REQUIRE(tile_mode == 1 || tile_rows, "latent_attn_tiles: tile_rows missing");
+    EXL2_REQUIRE(nsplit <= LA_MAX_SPLIT, "latent_attn_tiles: at most %d key splits", LA_MAX_SPLIT);
     EXL2_REQUIRE(nsplit >= 1 && (nsplit == 1 || (tile_mode == 1 && part_o && part_ml)), "latent_attn_tiles: key splits need tile_mode 1 and scratch");
     EXL2_REQUIRE(heads > 0 && page > 0 && window > 0 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent_attn_tiles: bad shape");
     if (kv_rank % 32 != 0 || kv_rank > 512 || kv_rank <= 0 || rot % 8 != 0 || rot > 32 * LA_ROT_STEPS)
@@ -522,16 +556,6 @@ extern "C" int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride,
     a.H = heads; a.R = kv_rank; a.rot = rot; a.rot_dims = rot_dims; a.inv_freq = inv_freq; a.scale = scale; a.window = window;
     a.DP = (kv_rank + rot + 31) / 32 * 32;
     const size_t smem = ((size_t)LA_KT * (a.DP + 8) + (size_t)kv_rank * LA_TS + 4 * 16 * LA_TS) * 2;
-    static bool attr_done[EXL2_MAX_DEVICES];
-    if (exl2_first_on_device(attr_done))
-    {
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<8, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<16, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<32, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<8, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<16, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        (void)hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<32, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    }
     hipStream_t s = (hipStream_t)stream;
     if (kv_rank <= 128) launch_lat_mfma<8>(a, tiles, tile_mode, smem, s);
     else if (kv_rank <= 256) launch_lat_mfma<16>(a, tiles, tile_mode, smem, s);

@@ -237,7 +237,8 @@ def test_latent_attention_random(be, dtype, R, rot, dims, H, window, page):
 
 
 @pytest.mark.parametrize("R,rot,dims,H,window,page,n", [(32, 8, 8, 3, 5, 4, 40), (64, 16, 8, 5, 37, 8, 75), (160, 8, 8, 17, 1000, 16, 70),
-                                                         (32, 40, 40, 70, 33, 7, 50), (288, 8, 4, 2, 20, 16, 45)])
+                                                         (32, 40, 40, 70, 33, 7, 50), (288, 8, 4, 2, 20, 16, 45), (128, 32, 32, 2, 40, 16, 70),
+                                                         (256, 64, 48, 5, 64, 32, 66)])
 @pytest.mark.parametrize("tiles", [(16, 1), (1, 1), (1, 3), (1, 8)])
 def test_latent_attention_on_the_matrix_cores(be, R, rot, dims, H, window, page, n, tiles):
     """the bfloat16 tile kernels (portions: 16 positions x a head per wave; decoded tokens: a position x 16 heads per wave, keys split
