@@ -1,6 +1,6 @@
 """Model registry: config.json's architecture name -> (configuration reader, model class, checkpoint adapter).
 
-`load_model(dir)` is how the command line, the trace runner and the benchmark get a model: it reads config.json, picks the entry,
+`load_model(dir)` is how the command line (generate, trace) and the benchmark get a model: it reads config.json, picks the entry,
 streams model.safetensors to the device (loader.py) and builds the modules."""
 from __future__ import annotations
 

@@ -42,9 +42,6 @@ def cmd_generate(a) -> int:
     from .engine import Engine, Generator
     model = load_model(a.model, device=a.device, dtype=_dtype(a.dtype))
     prompts = [[int(t) for t in s.replace(" ", "").split(",") if t] for s in a.tokens]
-    if not hasattr(model, "step"):
-        raise SystemExit("generate: this architecture is served through GreedyGraphDecoder (see bench.py); the paged engine "
-                         "takes models with a step() forward")
     need = sum(len(p) + a.max_new_tokens for p in prompts)
     eng = Engine(model, max_tokens=min(need, a.max_tokens) if a.max_tokens else need, max_seqs=a.max_seqs)
     out = Generator(eng, chunk=a.chunk).generate(prompts, a.max_new_tokens, temperature=a.temperature, top_k=a.top_k, top_p=a.top_p,

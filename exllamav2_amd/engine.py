@@ -25,7 +25,7 @@ class Engine:
         self.pool = PagePool(pages, page_size, max_seqs, model.device)
         self.cache = model.make_cache(self.pool)
         self.slots = {}                                           # request id -> slot
-        self.graphs = (model.device.type == "cuda") if graphs is None else bool(graphs)
+        self.graphs = ((model.device.type == "cuda") if graphs is None else bool(graphs)) and getattr(model, "graph_safe_step", False)
         self._decode = {}                                         # batch size -> captured decode step
         self._stream = torch.cuda.Stream(device=model.device) if self.graphs and model.device.type == "cuda" else None
 
@@ -41,6 +41,7 @@ class Engine:
         back after the step.  Returns fp32 logits [n wanted, vocab] on the device, or None."""
         ids, seq, pos, want_rows = [], [], [], []
         t16_row0, t16_rows, t1_row0, t1_maxpos = [], [], [], 0
+        spans = []
         seen = set()
         for rid, tokens, want in entries:
             if rid in seen:
@@ -54,6 +55,7 @@ class Engine:
             slot = self.slots[rid]
             start = self.pool.extend(slot, n)
             base = len(ids)
+            spans.append((base, n, slot, start))
             if n == 1:
                 t1_row0.append(base)
                 t1_maxpos = max(t1_maxpos, start)
@@ -75,7 +77,7 @@ class Engine:
             dev = self.model.device
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
-            batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows))
+            batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows), spans=spans)
             if t16_row0:
                 t16 = torch.tensor([t16_row0, t16_rows], dtype=torch.int32).to(dev)
                 batch.tiles16 = (t16[0], t16[1], len(t16_row0))

@@ -58,9 +58,13 @@ class StepBatch:
     # (row0 int32 [n], rows int32 [n], n) and single decoded tokens (row0 int32 [n], n, largest position among them)
     tiles16: tuple | None = None
     tiles1: tuple | None = None
+    # host-side view of the same rows, one tuple per request in the step: (first row, rows, sequence slot, first position)
+    spans: list | None = None
 
 
 class LayeredModel:
+    graph_safe_step = True                                # step() is launches on device-resident inputs only: an engine may capture it
+
     def __init__(self, config: LayeredConfig, device="cuda:0", dtype=torch.bfloat16, ext=None):
         if dtype not in (torch.bfloat16, torch.float32):
             raise RuntimeError("LayeredModel: operand dtype is bfloat16 or float32")

@@ -120,6 +120,39 @@ class ExLlamaV2:
                 n += per_expert * mlp.num_experts_per_token + mlp.gate.numel() * 2
         return n
 
+    # ---- the paged engine's interface (exllamav2_amd/engine.py) -----------------------------------------------------------
+
+    @property
+    def vocab(self) -> int:
+        return self.config.vocab_size
+
+    def make_cache(self, pool):
+        """an FP16 cache whose storage IS the pool's pages ([pages, 256, kv_heads, head_dim] per layer), reached through the pool's
+        block table like the dynamic generator's cache (attn.py:504-505)"""
+        from .cache import ExLlamaV2Cache
+        if pool.page_size != PAGE_SIZE:
+            raise RuntimeError(f"the quantized models' attention kernels address pages of {PAGE_SIZE} tokens")
+        return ExLlamaV2Cache(self, batch_size=pool.num_pages, max_seq_len=PAGE_SIZE)
+
+    def step(self, batch, cache):
+        """One engine step: every request's rows go through forward_chunk in paged mode (positions and pages read on the device);
+        returns fp32 logits of the wanted rows, in order."""
+        cfg = self.config
+        rows_out = []
+        for row0, n, slot, _start in batch.spans:
+            at = 0
+            while at < n:
+                m = min(self.max_rows, n - at)
+                ids = batch.ids[row0 + at:row0 + at + m].view(1, m)
+                seqlens = batch.row_pos[row0 + at:row0 + at + 1].contiguous()
+                table = batch.block_table[slot:slot + 1].contiguous()
+                rows_out.append(self.forward_chunk(ids, cache, 0, cache_seqlens=seqlens, block_table=table, last_id_only=False)
+                                .view(m, cfg.vocab_size))
+                at += m
+        if batch.n_logits == 0:
+            return None
+        return torch.cat(rows_out, 0).index_select(0, batch.logit_rows.long()).float()
+
     # ---- forward ------------------------------------------------------------------------------------------------------
 
     def forward_chunk(self, input_ids: torch.Tensor, cache, past_len: int = 0, cache_seqlens=None, block_table=None,

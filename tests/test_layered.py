@@ -505,3 +505,33 @@ def test_trace_command_replays_steps(tmp_path, dtype):
     assert rel_err(g1, wb[[7]]) <= tol
     g2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)
     assert rel_err(g2, np.stack([wb[8], wa[299]])) <= tol
+
+
+def test_engine_serves_the_quantized_family_too(be):
+    """the same Engine.step / Generator over a quantized Llama-style model: its paged forward behind the engine's interface gives
+    what its own contiguous-cache forward gives, in portions and decoding, two requests side by side"""
+    from exllamav2_amd import ExLlamaV2, ExLlamaV2Cache, ExLlamaV2Config
+    from exllamav2_amd.engine import Engine, Generator
+    from exllamav2_amd.synth import synth_checkpoint
+    cfg = ExLlamaV2Config.tiny_test(num_hidden_layers=2, max_seq_len=512, max_input_len=16)
+    model = ExLlamaV2(cfg, device=be.device, ext=be.ext).load(synth_checkpoint(cfg, be.device, seed=3))
+    rng = np.random.default_rng(3)
+    a, b = rng.integers(0, cfg.vocab_size, size=9), rng.integers(0, cfg.vocab_size, size=5)
+    want = {}
+    for name, ids in (("a", a), ("b", b)):
+        cache = ExLlamaV2Cache(model, batch_size=1)
+        want[name] = be.n(model.forward(torch.from_numpy(ids[None, :]), cache, last_id_only=False).float())[0]
+    eng = Engine(model, max_tokens=512, max_seqs=2)
+    got = {"a": [], "b": []}
+    for step in ([("a", 0, 4)], [("a", 4, 7), ("b", 0, 4)], [("a", 7, 8), ("b", 4, 5)], [("a", 8, 9)]):
+        lg = be.n(eng.step([(r, list(map(int, {"a": a, "b": b}[r][lo:hi])), list(range(hi - lo))) for r, lo, hi in step]))
+        k = 0
+        for r, lo, hi in step:
+            got[r].append(lg[k:k + hi - lo]); k += hi - lo
+    for r in ("a", "b"):
+        g = np.concatenate(got[r], 0)
+        assert np.abs(g - want[r]).max() <= 0.06 + np.abs(want[r]).max() * 2.0 ** -7, r
+    eng.finish("a"); eng.finish("b")
+    out = Generator(eng, chunk=4).generate([list(map(int, a[:6])), list(map(int, b))], 3)
+    assert [len(o) for o in out] == [3, 3]
+    model.unload()
