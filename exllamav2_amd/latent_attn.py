@@ -11,6 +11,8 @@ Everything the design leaves open is a constructor parameter: head count and the
 base / dims, score scale."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .dense_linear import DenseLinear
@@ -23,7 +25,7 @@ def rotary_inv_freq(base: float, dims: int, device) -> torch.Tensor:
 
 
 class LatentAttention:
-    KEYS_PER_SPLIT = 64                                   # decoded tokens: keys per workgroup of the split-key attention launch
+    KEYS_PER_SPLIT = int(os.environ.get("EXL2_LATENT_KEYS_PER_SPLIT", "64"))     # decoded tokens: keys per workgroup of the split-key launch
 
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: int,
                  window: int, rot_base: float, rot_dims: int, scale: float, kv_from: int | None = None):
