@@ -174,7 +174,8 @@ KERNEL void __launch_bounds__(256) latent_attn_kernel(const LatAttnArgs a)
 // portion; the four waves of a workgroup take four heads), TR = 1: one position x sixteen heads (a decoded token).  Keys go by in
 // steps of 32: the workgroup stages the step's cache rows in LDS twice -- row-major for S = Q C^T (both operands K-contiguous) and
 // transposed ([latent element][key]) for O += P C, whose B operand wants 8 consecutive KEYS of one latent element per lane.  The
-// scores leave the accumulators through a wave-private LDS tile to become the A operand of the second product.  Softmax state
+// scores leave the accumulators through a wave-private LDS tile (laid over the row-major copy once all waves have used it) to become
+// the A operand of the second product.  Softmax state
 // (running maximum, sum) is per query row = per accumulator row, kept in registers; fp32 throughout, P rounded to bfloat16 for the
 // matrix core.  grid.z > 1 splits the key steps over workgroups (decoding against a long window): partial (m, l, O) go to
 // scratch and latent_attn_merge_kernel joins them.
@@ -220,7 +221,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     const int D = R + rot, DP = RS > 0 ? D : a.DP, CS = DP + 8;
     u16* Cs = (u16*)smem;                                    // [32][CS]
     u16* Ct = Cs + LA_KT * CS;                               // [R][LA_TS]
-    u16* Ps = Ct + R * LA_TS + w * 16 * LA_TS;               // [16][LA_TS], this wave's
+    u16* Ps = Cs + w * 16 * LA_TS;                           // [16][LA_TS], this wave's: OVER the row-major copy, once every wave is done with it
 
     // the query vector this lane feeds as A-operand row li
     int qrow, qhead;
@@ -341,7 +342,7 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
             issue(row_next);
             if (st + 2 < s_end) row_next = key_row(st + 2);
         }
-        float corr[4];
+        float corr[4], pe0[4], pe1[4];
         if (wave_live)
         {
             f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -375,27 +376,45 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                 const float mx = row16_allreduce_max(fmaxf(v0, v1));
                 const float m_new = fmaxf(m_run[r], mx);
                 const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-                const float e0 = expf(v0 - m_safe), e1 = expf(v1 - m_safe);
-                corr[r] = expf(m_run[r] - m_safe);
+                const float e0 = fast_exp(v0 - m_safe), e1 = fast_exp(v1 - m_safe);     // (bfloat16 path: the hardware exponential)
+                corr[r] = fast_exp(m_run[r] - m_safe);
                 l_run[r] = l_run[r] * corr[r] + row16_allreduce_add(e0 + e1);
                 m_run[r] = m_new;
-                Ps[qi * LA_TS + li] = f32_to_bf16(e0);
-                Ps[qi * LA_TS + 16 + li] = f32_to_bf16(e1);
+                pe0[r] = e0; pe1[r] = e1;
+            }
+        }
+        block_sync_lds();                                 // every wave has read its S operands: the probability tiles may overwrite them
+        if (wave_live)
+        {
+            #pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                Ps[(4 * g + r) * LA_TS + li] = f32_to_bf16(pe0[r]);
+                Ps[(4 * g + r) * LA_TS + 16 + li] = f32_to_bf16(pe1[r]);
             }
         }
         block_sync_lds();
         if (wave_live)
         {
             const u32x4 pa = *(const u32x4*)(Ps + li * LA_TS + 8 * g);
+            // the running maxima rarely move once a few steps have gone by: rescale the accumulators only when one did
+            const bool moved = wave_ballot(corr[0] != 1.0f || corr[1] != 1.0f || corr[2] != 1.0f || corr[3] != 1.0f) != 0ull;
+            if (moved)
+            {
+                #pragma unroll
+                for (int nt = 0; nt < NT; nt++)
+                    if (nt * 16 < R)
+                    {
+                        #pragma unroll
+                        for (int r = 0; r < 4; r++) acc[nt][r] *= corr[r];
+                    }
+            }
             #pragma unroll
             for (int nt = 0; nt < NT; nt++)
                 if (nt * 16 < R)
                 {
-                    f32x4 o = acc[nt];
-                    #pragma unroll
-                    for (int r = 0; r < 4; r++) o[r] *= corr[r];
                     const u32x4 b = *(const u32x4*)(Ct + (nt * 16 + li) * LA_TS + 8 * g);
-                    acc[nt] = mfma_16x16x32_bf16(pa, b, o);
+                    acc[nt] = mfma_16x16x32_bf16(pa, b, acc[nt]);
                 }
         }
         block_sync_lds();
@@ -555,7 +574,7 @@ extern "C" int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride,
     a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.out = (u16*)out; a.part_o = part_o; a.part_ml = part_ml; a.nsplit = nsplit;
     a.H = heads; a.R = kv_rank; a.rot = rot; a.rot_dims = rot_dims; a.inv_freq = inv_freq; a.scale = scale; a.window = window;
     a.DP = (kv_rank + rot + 31) / 32 * 32;
-    const size_t smem = ((size_t)LA_KT * (a.DP + 8) + (size_t)kv_rank * LA_TS + 4 * 16 * LA_TS) * 2;
+    const size_t smem = ((size_t)LA_KT * (a.DP + 8) + (size_t)kv_rank * LA_TS) * 2;      // (<= 78 KB: two workgroups per CU)
     hipStream_t s = (hipStream_t)stream;
     if (kv_rank <= 128) launch_lat_mfma<8>(a, tiles, tile_mode, smem, s);
     else if (kv_rank <= 256) launch_lat_mfma<16>(a, tiles, tile_mode, smem, s);
