@@ -69,12 +69,20 @@ def random_tensors(cfg: dict, device, seed: int = 0) -> dict:
 
 
 def _timed(fn, reps: int):
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / reps
+    """seconds per call; the interpreter's cyclic collector is held off while the clock runs (a full collection of a process that has
+    imported torch takes tens of milliseconds and would land in one of a few repetitions)"""
+    import gc
+    gc.collect()
+    gc.disable()
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+    finally:
+        gc.enable()
 
 
 def bench_layered(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
