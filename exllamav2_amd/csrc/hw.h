@@ -405,6 +405,9 @@ DEV void* global_ptr_of(u32 lo, u32 hi)
 // fast math
 DEV float fast_exp(float x) { return __expf(x); }
 DEV float fast_rsqrt(float x) { return rsqrtf(x); }
+// hardware sine / cosine: for arguments already reduced to [-pi, pi]
+DEV float fast_sin(float x) { return __sinf(x); }
+DEV float fast_cos(float x) { return __cosf(x); }
 DEV float fast_rcp(float x) { return __frcp_rn(x); }
 
 // shader-clock timestamp (s_memtime): used only by the EXL2_TRACE profiling build

@@ -234,15 +234,28 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     constexpr int KSC = NT / 2;
     u32x4 qf[KSC + LA_ROT_STEPS];
     {
+        // (all loads of a batch of 8 k-steps first, then the conversions: a conversion right behind its load makes every k-step a
+        // memory round trip of its own)
         const float* qa = a.q_abs + ((long long)qrow * H + qh) * R;
         #pragma unroll
-        for (int ks = 0; ks < KSC; ks++)
+        for (int k0 = 0; k0 < KSC; k0 += 8)
         {
-            qf[ks] = (u32x4){0u, 0u, 0u, 0u};
-            if (ks * 32 < R)
+            f32x4 lo[8], hi[8];
+            #pragma unroll
+            for (int j = 0; j < 8; j++)
             {
-                const float* s = qa + ks * 32 + 8 * g;
-                qf[ks] = (u32x4){la_pack2(s[0], s[1]), la_pack2(s[2], s[3]), la_pack2(s[4], s[5]), la_pack2(s[6], s[7])};
+                const int ks = min(k0 + j, KSC - 1);
+                const int off = min(ks * 32, R - 32) + 8 * g;          // (clamped: k-steps past kv_rank re-read the last one and are zeroed below)
+                lo[j] = *(const f32x4*)(qa + off);
+                hi[j] = *(const f32x4*)(qa + off + 4);
+            }
+            #pragma unroll
+            for (int j = 0; j < 8; j++)
+            {
+                const int ks = k0 + j;
+                if (ks >= KSC) continue;
+                qf[ks] = ks * 32 < R ? (u32x4){la_pack2(lo[j][0], lo[j][1]), la_pack2(lo[j][2], lo[j][3]), la_pack2(hi[j][0], hi[j][1]), la_pack2(hi[j][2], hi[j][3])}
+                                     : (u32x4){0u, 0u, 0u, 0u};
             }
         }
         const u16* qr = a.q + (long long)qrow * a.ldq + (long long)qh * a.q_head_stride + a.q_rot_off;
@@ -262,8 +275,12 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                         x0 = bf16_to_f32(qr[i0]); x1 = bf16_to_f32(qr[i0 + 1]);
                         if (i0 < a.rot_dims)
                         {
+                            // (bfloat16 path: two-term reduction of the fp32 angle to [-pi, pi], then the hardware sine / cosine -- the
+                            // library functions' large-argument path costs microseconds per call in a prologue that runs once per key split)
                             const float ang = (float)qpos * a.inv_freq[i0 >> 1];
-                            const float c = cosf(ang), sn = sinf(ang);
+                            const float nrev = rintf(ang * 0.15915494309189535f);
+                            const float red = fmaf(-nrev, -1.7484555e-07f, fmaf(-nrev, 6.2831855f, ang));
+                            const float c = fast_cos(red), sn = fast_sin(red);
                             const float u = x0, vv = x1;
                             x0 = u * c - vv * sn; x1 = vv * c + u * sn;
                         }
@@ -294,9 +311,15 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
     const int skey = t & (LA_KT - 1), sch0 = t >> 5;
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     u32x4 sv[LA_STAGE_IT];
-    auto key_row = [&](int st) -> long long {
+    // the page of this thread's key in step st (a load) and, separately, the row offset made from it: the load is issued a whole step
+    // before its value is consumed, so no wait for it ever sits behind freshly issued row loads
+    auto key_page = [&](int st) -> int {
         const int j = min(k_lo + st * LA_KT + skey, k_hi);
-        return ((long long)bt[j / a.page] * a.page + j % a.page) * D;
+        return bt[j / a.page];
+    };
+    auto key_row = [&](int pg, int st) -> long long {
+        const int j = min(k_lo + st * LA_KT + skey, k_hi);
+        return ((long long)pg * a.page + j % a.page) * D;
     };
     auto issue = [&](long long rowoff) {
         #pragma unroll
@@ -325,11 +348,11 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
             }
         }
     };
-    long long row_next = 0;
+    int pg_next = 0;
     if (s_begin < s_end)
     {
-        issue(key_row(s_begin));
-        if (s_begin + 1 < s_end) row_next = key_row(s_begin + 1);
+        issue(key_row(key_page(s_begin), s_begin));
+        if (s_begin + 1 < s_end) pg_next = key_page(s_begin + 1);
     }
 
     for (int st = s_begin; st < s_end; st++)
@@ -339,22 +362,33 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
         block_sync_lds();                                 // (LDS-only barriers: the loads issued below stay in flight across them)
         if (st + 1 < s_end)
         {
-            issue(row_next);
-            if (st + 2 < s_end) row_next = key_row(st + 2);
+            issue(key_row(pg_next, st + 1));
+            if (st + 2 < s_end) pg_next = key_page(st + 2);
         }
         float corr[4], pe0[4], pe1[4];
         if (wave_live)
         {
             f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            // (operand reads in batches of four k-steps ahead of their products: one wave per SIMD has nobody else to hide LDS latency)
             #pragma unroll
-            for (int ks = 0; ks < KSC; ks++)
-                if (ks * 32 < R)
-                {
-                    const u32x4 b0 = *(const u32x4*)(Cs + li * CS + ks * 32 + 8 * g);
-                    const u32x4 b1 = *(const u32x4*)(Cs + (16 + li) * CS + ks * 32 + 8 * g);
-                    s0 = mfma_16x16x32_bf16(qf[ks], b0, s0);
-                    s1 = mfma_16x16x32_bf16(qf[ks], b1, s1);
-                }
+            for (int k0 = 0; k0 < KSC; k0 += 4)
+            {
+                u32x4 b0[4], b1[4];
+                #pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (k0 + j < KSC && (k0 + j) * 32 < R)
+                    {
+                        b0[j] = *(const u32x4*)(Cs + li * CS + (k0 + j) * 32 + 8 * g);
+                        b1[j] = *(const u32x4*)(Cs + (16 + li) * CS + (k0 + j) * 32 + 8 * g);
+                    }
+                #pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (k0 + j < KSC && (k0 + j) * 32 < R)
+                    {
+                        s0 = mfma_16x16x32_bf16(qf[k0 + j], b0[j], s0);
+                        s1 = mfma_16x16x32_bf16(qf[k0 + j], b1[j], s1);
+                    }
+            }
             #pragma unroll
             for (int ks = 0; ks < LA_ROT_STEPS; ks++)
                 if (ks * 32 < rot)
@@ -410,12 +444,16 @@ KERNEL void __launch_bounds__(256) latent_attn_mfma_kernel(const LatMfmaArgs a)
                     }
             }
             #pragma unroll
-            for (int nt = 0; nt < NT; nt++)
-                if (nt * 16 < R)
-                {
-                    const u32x4 b = *(const u32x4*)(Ct + (nt * 16 + li) * LA_TS + 8 * g);
-                    acc[nt] = mfma_16x16x32_bf16(pa, b, acc[nt]);
-                }
+            for (int n0 = 0; n0 < NT; n0 += 8)
+            {
+                u32x4 b[8];
+                #pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if ((n0 + j) * 16 < R) b[j] = *(const u32x4*)(Ct + ((n0 + j) * 16 + li) * LA_TS + 8 * g);
+                #pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if ((n0 + j) * 16 < R) acc[n0 + j] = mfma_16x16x32_bf16(pa, b[j], acc[n0 + j]);
+            }
         }
         block_sync_lds();
     }

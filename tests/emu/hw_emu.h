@@ -132,6 +132,8 @@ DEV f16x2 h2_dup(f16 x) { return (f16x2){x, x}; }
 
 DEV float fast_exp(float x) { return expf(x); }
 DEV float fast_rsqrt(float x) { return 1.0f / sqrtf(x); }
+DEV float fast_sin(float x) { return sinf(x); }
+DEV float fast_cos(float x) { return cosf(x); }
 DEV float fast_rcp(float x) { return 1.0f / x; }
 
 template <typename T> DEV void pin_scalar(T&) { }
