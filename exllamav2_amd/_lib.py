@@ -115,6 +115,14 @@ PROTOTYPES = {
     "exl2_latent_append": (ci, [vp, ci, vp, cf, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, ci, vp, vp]),
     "exl2_latent_attn": (ci, [vp, ci, ci, ci, vp, vp, ci, vp, vp, vp, ci, vp, ci, ci, ci, ci, ci, ci, vp, cf, ci, vp]),
     "exl2_latent_attn_tiles": (ci, [vp, ci, ci, ci, vp, vp, ci, vp, vp, vp, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, ci, ci, vp, cf, ci, vp]),
+    "exl2_dense_linear_bias": (ci, [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, cll, cll, cll, cll, vp, ci, vp, vp, vp, ci, ci, cf, vp]),
+    "exl2_add_layer_norm": (ci, [vp, vp, vp, vp, vp, ci, vp, ci, ci, ci, cf, vp]),
+    # state-space mixer (csrc/ssm.hip), windowed attention with pooled blocks (csrc/window_attn.hip)
+    "exl2_conv_silu_rows": (ci, [vp, ci, vp, vp, vp, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, vp]),
+    "exl2_ssm_scan": (ci, [vp, ci, vp, vp, ci, vp, ci, vp, vp, vp, vp, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, vp]),
+    "exl2_gated_group_norm": (ci, [vp, ci, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci, cf, vp]),
+    "exl2_kv_rot_append": (ci, [vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, vp, cf, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]),
+    "exl2_window_attn": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

@@ -174,3 +174,53 @@ class LatentCache:
 
     def footprint(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.rows.values())
+
+
+class PagedKV:
+    """One attention layer's share of a PagePool: keys [pages, page, kv_heads, dim] and values [pages, page, kv_heads, vdim], and --
+    for layers that see pooled blocks behind their window -- one mean key / mean value row per block of `block` tokens, kept with
+    the page of the block's first token: [pages, ceil(page / block), kv_heads, dim | vdim]."""
+
+    def __init__(self, pool: PagePool, kv_heads: int, dim: int, vdim: int, block: int, dtype):
+        dev, P, n = pool.device, pool.page_size, pool.num_pages
+        self.block = int(block)
+        self.k = torch.zeros((n, P, kv_heads, dim), dtype=dtype, device=dev)
+        self.v = torch.zeros((n, P, kv_heads, vdim), dtype=dtype, device=dev)
+        self.k_pool = self.v_pool = None
+        if self.block > 0:
+            per_page = -(-P // self.block)
+            self.k_pool = torch.zeros((n, per_page, kv_heads, dim), dtype=dtype, device=dev)
+            self.v_pool = torch.zeros((n, per_page, kv_heads, vdim), dtype=dtype, device=dev)
+
+    def tensors(self):
+        return [t for t in (self.k, self.v, self.k_pool, self.v_pool) if t is not None]
+
+
+class SlotState:
+    """One recurrent layer's state per sequence slot of a PagePool: named fp32 tensors [max_seqs, ...].  Nothing is cleared when a
+    slot is handed to a new sequence: the kernels start a sequence's first portion (position 0) from zeros by themselves."""
+
+    def __init__(self, pool: PagePool, shapes: dict):
+        self.t = {name: torch.zeros((pool.max_seqs,) + tuple(shape), dtype=torch.float32, device=pool.device)
+                  for name, shape in shapes.items()}
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self.t[name]
+
+    def tensors(self):
+        return list(self.t.values())
+
+
+class LayerStates:
+    """What a stack of unlike mixers keeps between steps: per layer whatever its mixer's `make_state(pool, dtype)` built (PagedKV for
+    attention, SlotState for recurrent mixers), all over ONE PagePool, so a request's pages and its slot are handed out and taken
+    back together."""
+
+    def __init__(self, pool: PagePool, per_layer: dict):
+        self.pool, self.per_layer = pool, dict(per_layer)
+
+    def layer(self, layer_idx: int):
+        return self.per_layer[layer_idx]
+
+    def footprint(self) -> int:
+        return sum(t.numel() * t.element_size() for st in self.per_layer.values() if st is not None for t in st.tensors())

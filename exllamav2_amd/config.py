@@ -63,6 +63,23 @@ class LayeredConfig:
     postln_alpha: float = 1.0
     embedding_scale: float = 1.0
     layers: list = field(default_factory=list)
+    residual: str = "post_rms"        # "post_rms": x <- rms_norm(alpha x + f(x)) (1 + w);  "pre_ln": x <- x + f(layer_norm(x))
+    tied_head: bool = False           # logits from the embedding table itself (no `head` tensor)
+    logit_softcap: float = 0.0        # > 0: logits <- c tanh(logits / c)
+
+    @staticmethod
+    def from_dict_prenorm(d: dict) -> "LayeredConfig":
+        """pre-norm stacks with layer norms (weight and bias), a tied output table and an optional soft cap on the logits"""
+        try:
+            cfg = LayeredConfig(architecture=str(d["architecture"]), vocab=int(d["vocab"]), width=int(d["width"]),
+                                norm_eps=float(d["norm"]["eps"]), embedding_scale=float(d["embedding"]["scale"]),
+                                layers=list(d["layers"]), residual="pre_ln", tied_head=True,
+                                logit_softcap=float(d.get("logit_softcap") or 0.0))
+        except KeyError as e:
+            raise RuntimeError(f"config.json: missing key {e}") from e
+        if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:
+            raise RuntimeError("config.json: vocab, width and layers must be given")
+        return cfg
 
     @staticmethod
     def from_dict(d: dict) -> "LayeredConfig":

@@ -12,16 +12,19 @@
 // A call may be batched over blockIdx.z (per-head projections: element offsets per batch for x, w, y, aux) or GROUPED (sparse MoE
 // at many rows: batch z = expert z multiplies the rows listed for it, counts and lists in device memory, no host round trip).
 // Epilogues fold the layer's elementwise steps into the producing linear: acc * sigmoid(aux) (output gate), silu(aux) * acc
-// (gated MLP), and the clamped gated unit min(aux, L) * sigmoid(1.702 min(aux, L)) * (clamp(acc, -L, L) + 1).
+// (gated MLP), the clamped gated unit min(aux, L) * sigmoid(1.702 min(aux, L)) * (clamp(acc, -L, L) + 1), relu(acc)^2 and the soft
+// cap L tanh(acc / L); a bias vector (fp32, one value per output column) is added to the accumulator first.
 #include "hw.h"
 #include "errors.h"
 
 enum { DENSE_BF16 = 0, DENSE_F32 = 1 };
-enum { EPI_NONE = 0, EPI_MUL_SIGMOID_AUX = 1, EPI_SILU_AUX_MUL = 2, EPI_CLAMPED_GLU = 3 };
+enum { EPI_NONE = 0, EPI_MUL_SIGMOID_AUX = 1, EPI_SILU_AUX_MUL = 2, EPI_CLAMPED_GLU = 3, EPI_RELU_SQUARED = 4, EPI_SOFT_CAP = 5 };
+#define EPI_READS_AUX(e) ((e) >= EPI_MUL_SIGMOID_AUX && (e) <= EPI_CLAMPED_GLU)
 
 struct LinArgs
 {
     const void* x; const void* w; void* y; const float* aux;
+    const float* bias;                       // [N] added to the accumulator before the epilogue (nullptr: none)
     int M, N, K;
     int ldx, ldw, ldy, ldaux;
     long long sxb, swb, syb, sauxb;          // element offsets per batch (blockIdx.z)
@@ -73,6 +76,8 @@ DEV float lin_epilogue(int epi, float acc, float aux, float limit)
         const float u = fminf(fmaxf(acc, -limit), limit);
         return g * sigmoid_f32(1.702f * g) * (u + 1.0f);
     }
+    if (epi == EPI_RELU_SQUARED) { const float r = fmaxf(acc, 0.0f); return r * r; }
+    if (epi == EPI_SOFT_CAP) return limit * tanhf(acc / limit);
     return acc;
 }
 
@@ -140,8 +145,8 @@ KERNEL void __launch_bounds__(256) lin_rows_kernel(const LinArgs a)
             const int r = r0 + m;
             if (r >= a.M) break;
             float aux = 0.0f;
-            if (a.epi != EPI_NONE) aux = a.aux[(long long)z * a.sauxb + (long long)r * a.ldaux + n];
-            st1<TY>((TY*)a.y + (long long)z * a.syb + (long long)r * a.ldy + n, lin_epilogue(a.epi, acc[m], aux, a.limit));
+            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + (long long)r * a.ldaux + n];
+            st1<TY>((TY*)a.y + (long long)z * a.syb + (long long)r * a.ldy + n, lin_epilogue(a.epi, acc[m] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
         }
     }
 }
@@ -209,8 +214,8 @@ KERNEL void __launch_bounds__(256) lin_tile_kernel(const LinArgs a)
             const int n = n0 + tx * 4 + j;
             if (n >= a.N) continue;
             float aux = 0.0f;
-            if (a.epi != EPI_NONE) aux = a.aux[(long long)z * a.sauxb + r * a.ldaux + n];
-            st1<TY>((TY*)a.y + (long long)z * a.syb + r * a.ldy + n, lin_epilogue(a.epi, acc[i][j], aux, a.limit));
+            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + r * a.ldaux + n];
+            st1<TY>((TY*)a.y + (long long)z * a.syb + r * a.ldy + n, lin_epilogue(a.epi, acc[i][j] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
         }
     }
 }
@@ -279,8 +284,8 @@ KERNEL void __launch_bounds__(256) lin_mfma_kernel(const LinArgs a)
                 const int n = n0 + 16 * j + li;
                 if (n >= a.N) continue;
                 float aux = 0.0f;
-                if (a.epi != EPI_NONE) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
-                st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r], aux, a.limit));
+                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
+                st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
             }
         }
 }
@@ -376,8 +381,8 @@ KERNEL void __launch_bounds__(256) lin_mfma_tile_kernel(const LinArgs a)
                 const int n = n0 + wn + 16 * j + li;
                 if (n >= a.N) continue;
                 float aux = 0.0f;
-                if (a.epi != EPI_NONE) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
-                st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r], aux, a.limit));
+                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
+                st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
             }
         }
 }
@@ -415,24 +420,42 @@ static void launch_dense(const LinArgs& a, int batch, bool vec_ok, int max_rows,
     LAUNCH((lin_tile_kernel<T, TY>), dim3((a.N + 63) / 64, (max_rows + 63) / 64, batch), dim3(256), 0, s, a);
 }
 
+extern "C" int exl2_dense_linear_bias(const void* x, const void* w, const float* bias, void* y, const float* aux, int dtype, int y_f32,
+                                      int M, int N, int K, int ldx, int ldw, int ldy, int ldaux,
+                                      int batch, long long sxb, long long swb, long long syb, long long sauxb,
+                                      const int* w_sel, int n_sel, const int* grp_count, const int* grp_offset, const int* grp_rows,
+                                      int x_div, int epi, float limit, void* stream);
+
 extern "C" int exl2_dense_linear(const void* x, const void* w, void* y, const float* aux, int dtype, int y_f32,
                                  int M, int N, int K, int ldx, int ldw, int ldy, int ldaux,
                                  int batch, long long sxb, long long swb, long long syb, long long sauxb,
                                  const int* w_sel, int n_sel, const int* grp_count, const int* grp_offset, const int* grp_rows,
                                  int x_div, int epi, float limit, void* stream)
 {
+    return exl2_dense_linear_bias(x, w, nullptr, y, aux, dtype, y_f32, M, N, K, ldx, ldw, ldy, ldaux, batch, sxb, swb, syb, sauxb,
+                                  w_sel, n_sel, grp_count, grp_offset, grp_rows, x_div, epi, limit, stream);
+}
+
+extern "C" int exl2_dense_linear_bias(const void* x, const void* w, const float* bias, void* y, const float* aux, int dtype, int y_f32,
+                                      int M, int N, int K, int ldx, int ldw, int ldy, int ldaux,
+                                      int batch, long long sxb, long long swb, long long syb, long long sauxb,
+                                      const int* w_sel, int n_sel, const int* grp_count, const int* grp_offset, const int* grp_rows,
+                                      int x_div, int epi, float limit, void* stream)
+{
     EXL2_REQUIRE(x && w && y, "dense_linear: null operand");
     EXL2_REQUIRE(dtype == DENSE_BF16 || dtype == DENSE_F32, "dense_linear: dtype must be 0 (bfloat16) or 1 (float32)");
     EXL2_REQUIRE(M >= 0 && N > 0 && K > 0 && batch > 0 && x_div > 0, "dense_linear: bad shape %d x %d x %d, batch %d", M, N, K, batch);
     EXL2_REQUIRE(ldx >= K || x_div > 0, "dense_linear: ldx"); EXL2_REQUIRE(ldw >= K && ldy > 0, "dense_linear: leading dimensions");
-    EXL2_REQUIRE(epi >= EPI_NONE && epi <= EPI_CLAMPED_GLU, "dense_linear: unknown epilogue %d", epi);
-    EXL2_REQUIRE(epi == EPI_NONE || aux, "dense_linear: the epilogue needs aux");
+    EXL2_REQUIRE(epi >= EPI_NONE && epi <= EPI_SOFT_CAP, "dense_linear: unknown epilogue %d", epi);
+    EXL2_REQUIRE(!EPI_READS_AUX(epi) || aux, "dense_linear: the epilogue needs aux");
+    EXL2_REQUIRE(epi != EPI_SOFT_CAP || limit > 0.0f, "dense_linear: the soft cap needs a positive limit");
+    EXL2_REQUIRE(!bias || (batch == 1 && !w_sel && !grp_count), "dense_linear: a bias goes with a plain (one-slab) call");
     EXL2_REQUIRE(!(w_sel && grp_count), "dense_linear: w_sel and groups exclude each other");
     EXL2_REQUIRE(!grp_count || (grp_offset && grp_rows), "dense_linear: grouped call without offsets / row lists");
     EXL2_REQUIRE(dtype == DENSE_BF16 || y_f32, "dense_linear: float32 operands give float32 results");
     if (M == 0) return EXL2_OK;
     LinArgs a;
-    a.x = x; a.w = w; a.y = y; a.aux = aux; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.ldaux = ldaux;
+    a.x = x; a.w = w; a.y = y; a.aux = aux; a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldy = ldy; a.ldaux = ldaux;
     a.sxb = sxb; a.swb = swb; a.syb = syb; a.sauxb = sauxb; a.w_sel = w_sel; a.n_sel = n_sel;
     a.grp_count = grp_count; a.grp_offset = grp_offset; a.grp_rows = grp_rows; a.x_div = x_div; a.epi = epi; a.limit = limit;
     const int es = dtype == DENSE_BF16 ? 2 : 4, v = 16 / es;

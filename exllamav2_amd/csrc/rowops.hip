@@ -1,6 +1,7 @@
 // rowops.hip -- the row-wise steps around the dense linears (dense.hip), fp32 arithmetic throughout, + their C ABI:
 //   * embedding gather times a scale into the fp32 residual stream (+ its operand-dtype copy for the next linear),
 //   * RMS norm of a (strided) fp32 row slice with a plain weight w or a zero-centred one (1 + w), optional row gather,
+//   * the pre-norm residual step  x <- x + y  with the layer norm (weight and bias) that feeds the next sublayer,
 //   * the post-norm residual step  x <- norm(alpha x + y) (1 + w), where y is a linear's fp32 output or the weighted sum of a
 //     token's chosen experts (identity experts contribute the token's own x),
 //   * the sparse-MoE router (softmax over all experts, selection by score + correction, weights from the uncorrected scores) and
@@ -110,6 +111,48 @@ KERNEL void __launch_bounds__(256) post_norm_kernel(const PostNormArgs a)
         const float o = v[i] * rinv * (1.0f + ro_ld<T>((const T*)a.w + i));
         xr[i] = o;
         if (xh && (void*)xh != (void*)a.x) ro_st<T>(xh + (long long)r * a.width + i, o);
+    }
+}
+
+// ---- x <- x + y, then layer norm (mean removed, weight and bias) -------------------------------------------------------------------
+// The residual step of a pre-norm layer and the norm in front of the next sublayer as one launch: the fp32 stream takes the
+// sublayer's output (y, nullable), and the normalised row goes out in the operand dtype (w nullable: only the addition).  The
+// variance is the mean of the squared deviations from the mean (two passes over the row held in LDS).
+
+struct LayerNormArgs
+{
+    float* x; const float* y; const void* w; const void* b; void* out; int out_f32;
+    const int* row_idx;                      // nullable: output row r is made from stream row row_idx[r] (no addition then)
+    int width; float eps;
+};
+
+template <typename T>
+KERNEL void __launch_bounds__(256) add_layer_norm_kernel(const LayerNormArgs a)
+{
+    DYN_SMEM(smem);
+    SHARED float part[4];
+    float* v = (float*)smem;
+    const int r = bid_x();
+    const long long src = a.row_idx ? a.row_idx[r] : r;
+    float* xr = a.x + src * a.width;
+    float s = 0.0f;
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        float xv = xr[i];
+        if (a.y) { xv += a.y[src * a.width + i]; xr[i] = xv; }
+        v[i] = xv;
+        s += xv;
+    }
+    if (!a.w) return;
+    const float mean = block_sum_256(s, part) / (float)a.width;
+    float ss = 0.0f;
+    for (int i = tid(); i < a.width; i += 256) { const float d = v[i] - mean; ss = fmaf(d, d, ss); }
+    ss = block_sum_256(ss, part);
+    const float rinv = 1.0f / sqrtf(ss / (float)a.width + a.eps);
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        const float o = (v[i] - mean) * rinv * ro_ld<T>((const T*)a.w + i) + (a.b ? ro_ld<T>((const T*)a.b + i) : 0.0f);
+        if (a.out_f32) ((float*)a.out)[(long long)r * a.width + i] = o; else ro_st<T>((T*)a.out + (long long)r * a.width + i, o);
     }
 }
 
@@ -266,6 +309,34 @@ extern "C" int exl2_post_norm(float* x, void* xh, const float* y, const void* w,
     }
     if (dtype == 0) LAUNCH(post_norm_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
     else LAUNCH(post_norm_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_add_layer_norm(float* x, const float* y, const void* w, const void* b, void* out, int out_f32, const int* row_idx,
+                                   int dtype, int rows, int width, float eps, void* stream)
+{
+    EXL2_REQUIRE(x, "add_layer_norm: null stream");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "add_layer_norm: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(!w || out, "add_layer_norm: a norm needs an output");
+    EXL2_REQUIRE(w || y, "add_layer_norm: neither an addition nor a norm");
+    EXL2_REQUIRE(!(row_idx && y), "add_layer_norm: gathered rows take no addition");
+    EXL2_REQUIRE(width > 0 && (size_t)width * 4 <= 160 * 1024 - 64, "add_layer_norm: row of %d values does not fit the LDS", width);
+    if (rows <= 0) return EXL2_OK;
+    LayerNormArgs a;
+    a.x = x; a.y = y; a.w = w; a.b = b; a.out = out; a.out_f32 = out_f32 || dtype == 1; a.row_idx = row_idx; a.width = width; a.eps = eps;
+    const size_t smem = (size_t)width * 4;
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)add_layer_norm_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)add_layer_norm_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    if (dtype == 0) LAUNCH(add_layer_norm_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
+    else LAUNCH(add_layer_norm_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

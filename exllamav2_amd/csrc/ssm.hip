@@ -1,0 +1,302 @@
+// ssm.hip -- the recurrent half of a state-space mixer (selective scan with one scalar decay per head) for gfx950, + its C ABI:
+//   * the short causal convolution per channel with its bias and SiLU, over rows that continue a sequence (the last taps - 1
+//     inputs of every sequence are kept per slot),
+//   * the scan  S <- exp(-exp(A) dt) S + dt B u^T,  y = S^T C + D u  per head over the rows of each sequence's portion, with
+//     dt = softplus(dt_raw + dt_bias); the state S [state, vdim] is fp32 and lives per (slot, head),
+//   * the gate and the group-wise RMS norm  out = rms_g(y * silu(z)) * w.
+// Rows of a step are a flat list; a SPAN is the run of consecutive rows that one sequence brings (span i = rows span_row0[i] ..
+// + span_rows[i], its slot and first position are row_seq / row_pos of its first row).  A span that starts at position 0 starts
+// from a zero state and zero convolution history whatever its slot held before, so slots need no clearing when they are reused.
+// All arithmetic is fp32; inputs are the fp32 outputs of the mixer's input projection.
+#include "hw.h"
+#include "errors.h"
+
+template <typename T> DEV float ss_ld(const T* p);
+template <> DEV float ss_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
+template <> DEV float ss_ld<float>(const float* p) { return *p; }
+template <typename T> DEV void ss_st(T* p, float v);
+template <> DEV void ss_st<u16>(u16* p, float v) { *p = f32_to_bf16(v); }
+template <> DEV void ss_st<float>(float* p, float v) { *p = v; }
+
+DEV float ss_silu(float z) { return z / (1.0f + expf(-z)); }
+DEV float ss_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+// ---- causal convolution + SiLU ------------------------------------------------------------------------------------------------
+
+#define CONV_MAX_TAPS 8
+#define CONV_TOKENS 32                       // consecutive rows of a span that one workgroup walks
+
+struct ConvArgs
+{
+    const float* in; int ld;                 // [rows, ld]: the channels start at the pointer
+    const void* w; const void* bias;         // [channels, taps], [channels]
+    float* out; int ldo;                     // [rows, ldo]
+    float* tail;                             // [slots, taps - 1, channels]: inputs of the last taps - 1 positions of every sequence
+    const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
+    int channels, taps;
+};
+
+// grid (channel blocks, token chunks, spans): thread = one channel over CONV_TOKENS consecutive rows, the window of the last
+// taps inputs slides through registers.  Inputs in front of the span come from the slot's tail, inputs in front of the
+// sequence are zero.
+template <typename T>
+KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
+{
+    const int c = bid_x() * 256 + tid();
+    const int sp = bid_z();
+    const int n = a.span_rows[sp];
+    const int t0 = bid_y() * CONV_TOKENS;
+    if (c >= a.channels || t0 >= n) return;
+    const int r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    const float* tail = a.tail + (long long)a.row_seq[r0] * (a.taps - 1) * a.channels;
+    float w[CONV_MAX_TAPS], win[CONV_MAX_TAPS];
+    #pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS; k++) w[k] = k < a.taps ? ss_ld<T>((const T*)a.w + (long long)c * a.taps + k) : 0.0f;
+    const float bias = a.bias ? ss_ld<T>((const T*)a.bias + c) : 0.0f;
+    // win[k] = input at token t - (taps - 1) + k; tokens are counted within the span, token -d is position pos0 - d
+    #pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS; k++)
+    {
+        win[k] = 0.0f;
+        if (k >= 1 && k < a.taps)                                  // slot k of the next window = token t0 - (taps - 1) + (k - 1) + ... set below
+        {
+            const int tok = t0 - (a.taps - 1) + (k - 1);
+            if (tok >= 0) win[k] = a.in[(long long)(r0 + tok) * a.ld + c];
+            else if (pos0 + tok >= 0) win[k] = tail[(long long)(a.taps - 1 + tok) * a.channels + c];
+        }
+    }
+    const int t1 = min(n, t0 + CONV_TOKENS);
+    for (int t = t0; t < t1; t++)
+    {
+        #pragma unroll
+        for (int k = 0; k < CONV_MAX_TAPS - 1; k++) win[k] = win[k + 1];
+        // after the shift the newest value belongs at index taps - 1
+        const float cur = a.in[(long long)(r0 + t) * a.ld + c];
+        float acc = bias;
+        #pragma unroll
+        for (int k = 0; k < CONV_MAX_TAPS; k++)
+        {
+            if (k == a.taps - 1) win[k] = cur;
+            if (k < a.taps) acc = fmaf(w[k], win[k], acc);
+        }
+        a.out[(long long)(r0 + t) * a.ldo + c] = ss_silu(acc);
+    }
+}
+
+// The tails after the step: for every span the inputs of its last taps - 1 positions (rows of the span where it is long enough,
+// the old tail shifted where it is not).  One thread per (span, channel) reads all it needs before it writes.
+KERNEL void __launch_bounds__(256) conv_tail_kernel(const ConvArgs a)
+{
+    const int c = bid_x() * 256 + tid();
+    const int sp = bid_y();
+    if (c >= a.channels) return;
+    const int n = a.span_rows[sp], r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    float* tail = a.tail + (long long)a.row_seq[r0] * (a.taps - 1) * a.channels;
+    float nv[CONV_MAX_TAPS];
+    #pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS - 1; k++)
+    {
+        nv[k] = 0.0f;
+        if (k < a.taps - 1)
+        {
+            const int tok = n - (a.taps - 1) + k;                   // token of the span that lands in tail slot k
+            if (tok >= 0) nv[k] = a.in[(long long)(r0 + tok) * a.ld + c];
+            else if (pos0 + tok >= 0) nv[k] = tail[(long long)(a.taps - 1 + tok) * a.channels + c];
+        }
+    }
+    #pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS - 1; k++)
+        if (k < a.taps - 1) tail[(long long)k * a.channels + c] = nv[k];
+}
+
+// ---- selective scan -------------------------------------------------------------------------------------------------------------
+
+#define SCAN_CHUNK 16                        // tokens staged in LDS per round
+#define SCAN_MAX_NPT 64                      // state rows per thread
+
+struct ScanArgs
+{
+    const float* u; int ldu;                 // [rows, ldu]: head h's inputs at h * vdim
+    const float* B; const float* C; int ldbc; // [rows, ldbc]: group g's vectors at g * state
+    const float* dt; int lddt;               // [rows, lddt]: raw step sizes, head h at h
+    const float* dt_bias; const float* A_log; const float* D;       // [heads]
+    float* y; int ldy;                       // [rows, ldy]
+    float* state;                            // [slots, heads, state, vdim]
+    const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
+    int heads, groups, N, P, KS;             // KS = threads that share a column of the state (blockDim = P * KS)
+};
+
+// Workgroup = one (span, head), P * KS threads (+ idle ones up to a whole wave): thread (j, p) holds rows n = j, j + KS, .. of column p of the state in registers
+// for the whole span.  Tokens are taken SCAN_CHUNK at a time: their u, B, C, step size and decay are staged in LDS, every thread
+// steps its rows through the chunk keeping one partial dot product per token, and the partial sums of a column's KS threads
+// are added at the chunk's end (two barriers per chunk, none per token).
+template <int NPT>
+KERNEL void __launch_bounds__(256) scan_kernel(const ScanArgs a)
+{
+    DYN_SMEM(smem);
+    const int h = bid_x(), sp = bid_y();
+    const int n_tok = a.span_rows[sp], r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    const int g = h / (a.heads / a.groups);
+    const int P = a.P, N = a.N, KS = a.KS;
+    const int t = tid(), nt = nthreads();                      // P * KS rounded up to whole waves: the rest only help staging
+    const bool owner = t < P * KS;
+    const int p = t % P, j = t / P;
+    float* s_u = (float*)smem;                                   // [CHUNK, P]
+    float* s_B = s_u + SCAN_CHUNK * P;                           // [CHUNK, N]
+    float* s_C = s_B + SCAN_CHUNK * N;                           // [CHUNK, N]
+    float* s_dt = s_C + SCAN_CHUNK * N;                          // [CHUNK] step size, [CHUNK] decay
+    float* s_part = s_dt + 2 * SCAN_CHUNK;                       // [CHUNK, KS, P]
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
+    float S[NPT];
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
+    }
+    const float neg_a = -expf(a.A_log[h]), dtb = a.dt_bias[h], Dh = a.D[h];
+    for (int c0 = 0; c0 < n_tok; c0 += SCAN_CHUNK)
+    {
+        const int nc = min(SCAN_CHUNK, n_tok - c0);
+        block_sync();
+        for (int i = t; i < nc * P; i += nt) s_u[i] = a.u[(long long)(r0 + c0 + i / P) * a.ldu + h * P + i % P];
+        for (int i = t; i < nc * N; i += nt)
+        {
+            const long long row = r0 + c0 + i / N;
+            s_B[i] = a.B[row * a.ldbc + g * N + i % N];
+            s_C[i] = a.C[row * a.ldbc + g * N + i % N];
+        }
+        if (t < nc)
+        {
+            const float d = ss_softplus(a.dt[(long long)(r0 + c0 + t) * a.lddt + h] + dtb);
+            s_dt[t] = d;
+            s_dt[SCAN_CHUNK + t] = expf(neg_a * d);
+        }
+        block_sync();
+        for (int k = 0; owner && k < nc; k++)
+        {
+            const float d = s_dt[k], decay = s_dt[SCAN_CHUNK + k];
+            const float du = d * s_u[k * P + p];
+            float part = 0.0f;
+            #pragma unroll
+            for (int i = 0; i < NPT; i++)
+            {
+                const int n = j + KS * i;
+                if (n < N)
+                {
+                    S[i] = fmaf(decay, S[i], du * s_B[k * N + n]);
+                    part = fmaf(S[i], s_C[k * N + n], part);
+                }
+            }
+            s_part[(k * KS + j) * P + p] = part;
+        }
+        block_sync();
+        for (int i = t; i < nc * P; i += nt)
+        {
+            const int k = i / P, pp = i % P;
+            float yv = 0.0f;
+            for (int jj = 0; jj < KS; jj++) yv += s_part[(k * KS + jj) * P + pp];
+            a.y[(long long)(r0 + c0 + k) * a.ldy + h * P + pp] = fmaf(Dh, s_u[k * P + pp], yv);
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        if (owner && n < N) st[(long long)n * P + p] = S[i];
+    }
+}
+
+// ---- gate + group-wise RMS norm -------------------------------------------------------------------------------------------------
+
+// grid (rows, norm groups): out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part]
+template <typename T>
+KERNEL void __launch_bounds__(256) gated_group_norm_kernel(const float* y, int ldy, const float* z, int ldz, const T* w, void* out, int ldo,
+                                                            int out_f32, int part, float eps)
+{
+    SHARED float red[4];
+    const int r = bid_x(), o0 = bid_y() * part;
+    float ss = 0.0f;
+    for (int i = tid(); i < part; i += 256)
+    {
+        const float v = y[(long long)r * ldy + o0 + i] * ss_silu(z[(long long)r * ldz + o0 + i]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_allreduce_add(ss);
+    if (lane_id() == 0) red[wave_id()] = ss;
+    block_sync();
+    const float rinv = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)part + eps);
+    for (int i = tid(); i < part; i += 256)
+    {
+        const float v = y[(long long)r * ldy + o0 + i] * ss_silu(z[(long long)r * ldz + o0 + i]) * rinv * ss_ld<T>(w + o0 + i);
+        if (out_f32) ((float*)out)[(long long)r * ldo + o0 + i] = v; else ss_st<T>((T*)out + (long long)r * ldo + o0 + i, v);
+    }
+}
+
+// ---- C ABI ----------------------------------------------------------------------------------------------------------------------
+
+extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const void* bias, float* out, int ldo, float* tail,
+                                   const int* span_row0, const int* span_rows, int spans, int max_span_rows, const int* row_seq,
+                                   const int* row_pos, int dtype, int channels, int taps, void* stream)
+{
+    EXL2_REQUIRE(in && w && out && tail && span_row0 && span_rows && row_seq && row_pos, "conv_silu_rows: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "conv_silu_rows: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "conv_silu_rows: %d taps (1 .. %d)", taps, CONV_MAX_TAPS);
+    EXL2_REQUIRE(channels > 0 && ld >= channels && ldo >= channels, "conv_silu_rows: bad shape");
+    if (spans <= 0 || max_span_rows <= 0) return EXL2_OK;
+    ConvArgs a;
+    a.in = in; a.ld = ld; a.w = w; a.bias = bias; a.out = out; a.ldo = ldo; a.tail = tail; a.span_row0 = span_row0; a.span_rows = span_rows;
+    a.row_seq = row_seq; a.row_pos = row_pos; a.channels = channels; a.taps = taps;
+    const dim3 grid((channels + 255) / 256, (max_span_rows + CONV_TOKENS - 1) / CONV_TOKENS, spans);
+    if (dtype == 0) LAUNCH(conv_silu_kernel<u16>, grid, dim3(256), 0, stream, a);
+    else LAUNCH(conv_silu_kernel<float>, grid, dim3(256), 0, stream, a);
+    if (taps > 1) LAUNCH(conv_tail_kernel, dim3((channels + 255) / 256, spans), dim3(256), 0, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_ssm_scan(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
+                             const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
+                             const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
+                             int heads, int groups, int n_state, int vdim, void* stream)
+{
+    EXL2_REQUIRE(u && B && C && dt && dt_bias && A_log && D && y && state && span_row0 && span_rows && row_seq && row_pos,
+                 "ssm_scan: null operand");
+    EXL2_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0, "ssm_scan: %d heads in %d groups", heads, groups);
+    EXL2_REQUIRE(n_state > 0 && vdim > 0 && vdim <= 256, "ssm_scan: state %d x %d", n_state, vdim);
+    if (spans <= 0) return EXL2_OK;
+    int ks = 256 / vdim;
+    if (ks < 1) ks = 1;
+    if (ks > n_state) ks = n_state;
+    const int npt = (n_state + ks - 1) / ks;
+    EXL2_REQUIRE(npt <= SCAN_MAX_NPT, "ssm_scan: state %d x %d needs %d rows per thread (at most %d)", n_state, vdim, npt, SCAN_MAX_NPT);
+    ScanArgs a;
+    a.u = u; a.ldu = ldu; a.B = B; a.C = C; a.ldbc = ldbc; a.dt = dt; a.lddt = lddt; a.dt_bias = dt_bias; a.A_log = A_log; a.D = D;
+    a.y = y; a.ldy = ldy; a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.groups = groups; a.N = n_state; a.P = vdim; a.KS = ks;
+    const size_t smem = sizeof(float) * ((size_t)SCAN_CHUNK * (vdim + 2 * n_state + 2 + (size_t)ks * vdim));
+    EXL2_REQUIRE(smem <= 64 * 1024, "ssm_scan: state %d x %d does not fit the staging buffers", n_state, vdim);
+    const dim3 grid(heads, spans), block((vdim * ks + 63) / 64 * 64);
+    if (npt <= 8) LAUNCH(scan_kernel<8>, grid, block, smem, stream, a);
+    else if (npt <= 16) LAUNCH(scan_kernel<16>, grid, block, smem, stream, a);
+    else if (npt <= 32) LAUNCH(scan_kernel<32>, grid, block, smem, stream, a);
+    else LAUNCH(scan_kernel<SCAN_MAX_NPT>, grid, block, smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_gated_group_norm(const float* y, int ldy, const float* z, int ldz, const void* w, void* out, int ldo, int out_f32,
+                                     int dtype, int rows, int dim, int groups, float eps, void* stream)
+{
+    EXL2_REQUIRE(y && z && w && out, "gated_group_norm: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "gated_group_norm: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(dim > 0 && groups > 0 && dim % groups == 0, "gated_group_norm: %d values in %d groups", dim, groups);
+    if (rows <= 0) return EXL2_OK;
+    if (dtype == 0) LAUNCH(gated_group_norm_kernel<u16>, dim3(rows, groups), dim3(256), 0, stream, y, ldy, z, ldz, (const u16*)w, out, ldo, out_f32, dim / groups, eps);
+    else LAUNCH(gated_group_norm_kernel<float>, dim3(rows, groups), dim3(256), 0, stream, y, ldy, z, ldz, (const float*)w, out, ldo, 1, dim / groups, eps);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}

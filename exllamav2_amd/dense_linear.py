@@ -22,13 +22,13 @@ class DenseLinear:
         return self.weight.dtype
 
     def forward(self, x: torch.Tensor, rows: int, out_dtype=None, out: torch.Tensor | None = None, aux=None, epi: int = 0,
-                limit: float = 0.0, ldx: int | None = None, x_off: int = 0, aux_ld: int = 0, aux_off: int = 0) -> torch.Tensor:
-        """Plain call on the first `rows` rows of x (leading dimension ldx, first value at element x_off)."""
+                limit: float = 0.0, ldx: int | None = None, x_off: int = 0, aux_ld: int = 0, aux_off: int = 0, bias=None) -> torch.Tensor:
+        """Plain call on the first `rows` rows of x (leading dimension ldx, first value at element x_off); bias fp32 [out] or None."""
         n, k = self.out_features, self.in_features
         if out is None:
             out = torch.empty((rows, n), dtype=out_dtype or self.dtype, device=self.weight.device)
         self.ext.dense_linear(x, self.weight, out, rows, n, k, ldx or x.shape[-1], k, out.shape[-1], aux=aux, ldaux=aux_ld,
-                              epi=epi, limit=limit, x_off=x_off, aux_off=aux_off)
+                              epi=epi, limit=limit, x_off=x_off, aux_off=aux_off, bias=bias)
         return out
 
     def weight_bytes(self) -> int:

@@ -78,6 +78,8 @@ class Engine:
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
             batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows), spans=spans)
+            sp = torch.tensor([[s[0] for s in spans], [s[1] for s in spans]], dtype=torch.int32).to(dev)
+            batch.spans_dev = (sp[0], sp[1], len(spans), max(s[1] for s in spans))
             if t16_row0:
                 t16 = torch.tensor([t16_row0, t16_rows], dtype=torch.int32).to(dev)
                 batch.tiles16 = (t16[0], t16[1], len(t16_row0))
@@ -102,7 +104,7 @@ class Engine:
             st = {"inputs": torch.zeros((3, b), dtype=torch.int32, device=dev), "rows": ar, "graph": None, "runs": 0}
             cap = self.pool.num_pages * self.pool.page_size
             st["batch"] = StepBatch(st["inputs"][0], st["inputs"][1], st["inputs"][2], self.pool.device_table(), ar, b, b,
-                                    tiles1=(ar, b, cap - 1))
+                                    tiles1=(ar, b, cap - 1), spans_dev=(ar, torch.ones_like(ar), b, 1))
             self._decode[b] = st
         host = torch.tensor([ids, seq, pos], dtype=torch.int32)
         if self._stream is None:                                   # (no GPU: the same batch, eagerly)

@@ -777,7 +777,7 @@ class ExtC:
 
     # ---- unquantized models: dense linears, row-wise steps, latent attention (csrc/dense.hip, rowops.hip, latent_attn.hip) ------
 
-    EPI_NONE, EPI_MUL_SIGMOID_AUX, EPI_SILU_AUX_MUL, EPI_CLAMPED_GLU = 0, 1, 2, 3
+    EPI_NONE, EPI_MUL_SIGMOID_AUX, EPI_SILU_AUX_MUL, EPI_CLAMPED_GLU, EPI_RELU_SQUARED, EPI_SOFT_CAP = 0, 1, 2, 3, 4, 5
 
     @staticmethod
     def _dense_code(dtype) -> int:
@@ -789,9 +789,10 @@ class ExtC:
 
     def dense_linear(self, x, w, y, M: int, N: int, K: int, ldx: int, ldw: int, ldy: int, aux=None, ldaux: int = 0, batch: int = 1,
                      sxb: int = 0, swb: int = 0, syb: int = 0, sauxb: int = 0, w_sel=None, n_sel: int = 0, groups=None,
-                     x_div: int = 1, epi: int = 0, limit: float = 0.0, x_off: int = 0, y_off: int = 0, aux_off: int = 0) -> None:
-        """y = epilogue(x . w^T) on explicit shapes and strides (include/exl2_hip.h: exl2_dense_linear).  x / y / aux may be
-        views INTO larger buffers: *_off are element offsets of the first value.  groups = (count, offset, rows) int32 tensors."""
+                     x_div: int = 1, epi: int = 0, limit: float = 0.0, x_off: int = 0, y_off: int = 0, aux_off: int = 0, bias=None) -> None:
+        """y = epilogue(x . w^T + bias) on explicit shapes and strides (include/exl2_hip.h: exl2_dense_linear_bias).  x / y / aux may be
+        views INTO larger buffers: *_off are element offsets of the first value.  groups = (count, offset, rows) int32 tensors;
+        bias fp32 [N]."""
         code = self._dense_code(w.dtype)
         if x.dtype is not w.dtype:
             raise RuntimeError(f"dense_linear: x is {x.dtype}, w is {w.dtype}")
@@ -800,8 +801,10 @@ class ExtC:
         if batch == 1 and w_sel is None and groups is None and w.numel() < (N - 1) * ldw + K:
             raise RuntimeError("dense_linear: weight smaller than N x K")
         gc, go, gr = groups if groups is not None else (None, None, None)
-        self.lib.check(self.lib.exl2_dense_linear(
-            self._ptr(x, None, "x") + x_off * x.element_size(), self._ptr(w, None, "w"),
+        if bias is not None and bias.numel() != N:
+            raise RuntimeError(f"dense_linear: bias has {bias.numel()} values, N is {N}")
+        self.lib.check(self.lib.exl2_dense_linear_bias(
+            self._ptr(x, None, "x") + x_off * x.element_size(), self._ptr(w, None, "w"), self._ptr(bias, torch.float32, "bias"),
             self._ptr(y, None, "y") + y_off * y.element_size(),
             None if aux is None else self._ptr(aux, torch.float32, "aux") + aux_off * 4, code, int(y.dtype is torch.float32),
             int(M), int(N), int(K), int(ldx), int(ldw), int(ldy), int(ldaux), int(batch), int(sxb), int(swb), int(syb), int(sauxb),
@@ -882,6 +885,76 @@ class ExtC:
             self._ptr(tile_rows, torch.int32, "tile_rows"), int(tiles), int(tile_mode), self._ptr(part_o, torch.float32, "part_o"),
             self._ptr(part_ml, torch.float32, "part_ml"), int(nsplit), int(heads), int(kv_rank), int(rot), int(rot_dims),
             self._ptr(inv_freq, torch.float32, "inv_freq"), float(scale), int(window), self._stream(out)))
+
+    def add_layer_norm(self, x32, y, w, b, out, rows: int, eps: float, row_idx=None) -> None:
+        """x32[r] += y[r] (y may be None), then out[r] = layer_norm(x32[r]) * w + b (w None: only the addition); with row_idx output
+        row r is made from stream row row_idx[r]"""
+        width = x32.shape[-1]
+        code = self._dense_code(w.dtype) if w is not None else 1
+        self.lib.check(self.lib.exl2_add_layer_norm(self._ptr(x32, torch.float32, "x32"), self._ptr(y, torch.float32, "y"),
+                                                    self._ptr(w, None, "w"), self._ptr(b, None if w is None else w.dtype, "b"),
+                                                    self._ptr(out, None, "out"), int(out is not None and out.dtype is torch.float32),
+                                                    self._ptr(row_idx, torch.int32, "row_idx"), code, int(rows), int(width), float(eps),
+                                                    self._stream(x32)))
+
+    # ---- state-space mixer (csrc/ssm.hip) -------------------------------------------------------------------------------------------
+
+    def conv_silu_rows(self, f, ld: int, f_off: int, w, bias, out, tail, spans, row_seq, row_pos, channels: int, taps: int) -> None:
+        """spans = (span_row0 int32 [n], span_rows int32 [n], n, longest span); f fp32 [rows, ld], channels start at column f_off"""
+        row0, nrows, n, longest = spans
+        self.lib.check(self.lib.exl2_conv_silu_rows(self._ptr(f, torch.float32, "f") + f_off * 4, int(ld), self._ptr(w, None, "w"),
+                                                    self._ptr(bias, w.dtype, "bias"), self._ptr(out, torch.float32, "out"), out.shape[-1],
+                                                    self._ptr(tail, torch.float32, "tail"), self._ptr(row0, torch.int32, "span_row0"),
+                                                    self._ptr(nrows, torch.int32, "span_rows"), int(n), int(longest),
+                                                    self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+                                                    self._dense_code(w.dtype), int(channels), int(taps), self._stream(out)))
+
+    def ssm_scan(self, c, ldc: int, u_off: int, b_off: int, c_off: int, f, ldf: int, dt_off: int, dt_bias, a_log, d, y, state, spans,
+                 row_seq, row_pos, heads: int, groups: int, n_state: int, vdim: int) -> None:
+        """c fp32 [rows, ldc]: convolved u at u_off, B at b_off, C at c_off; raw step sizes in f fp32 [rows, ldf] at dt_off"""
+        row0, nrows, n, _longest = spans
+        cp, fp = self._ptr(c, torch.float32, "c"), self._ptr(f, torch.float32, "f")
+        self.lib.check(self.lib.exl2_ssm_scan(cp + u_off * 4, int(ldc), cp + b_off * 4, cp + c_off * 4, int(ldc), fp + dt_off * 4, int(ldf),
+                                              self._ptr(dt_bias, torch.float32, "dt_bias"), self._ptr(a_log, torch.float32, "A_log"),
+                                              self._ptr(d, torch.float32, "D"), self._ptr(y, torch.float32, "y"), y.shape[-1],
+                                              self._ptr(state, torch.float32, "state"), self._ptr(row0, torch.int32, "span_row0"),
+                                              self._ptr(nrows, torch.int32, "span_rows"), int(n), self._ptr(row_seq, torch.int32, "row_seq"),
+                                              self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(groups), int(n_state), int(vdim),
+                                              self._stream(y)))
+
+    def gated_group_norm(self, y, z, ldz: int, w, out, rows: int, dim: int, groups: int, eps: float) -> None:
+        """out = rms_per_group(y * silu(z)) * w; y fp32 [rows, dim], z fp32 rows of leading dimension ldz (first dim columns)"""
+        self.lib.check(self.lib.exl2_gated_group_norm(self._ptr(y, torch.float32, "y"), y.shape[-1], self._ptr(z, torch.float32, "z"), int(ldz),
+                                                      self._ptr(w, None, "w"), self._ptr(out, None, "out"), out.shape[-1],
+                                                      int(out.dtype is torch.float32), self._dense_code(w.dtype), int(rows), int(dim),
+                                                      int(groups), float(eps), self._stream(out)))
+
+    # ---- windowed attention with pooled blocks (csrc/window_attn.hip) ------------------------------------------------------------------
+
+    def kv_rot_append(self, f, ld: int, q_off: int, k_off: int, v_off: int, q_out, q_scale, k_cache, v_cache, k_pool, v_pool, freq,
+                      amp: float, rot_dims: int, vfreq, v_rot: bool, interleaved: bool, row_seq, row_pos, block_table, page: int, pool: int,
+                      rows: int, heads: int, kv_heads: int, dim: int, vdim: int) -> None:
+        dt = k_cache.dtype
+        self.lib.check(self.lib.exl2_kv_rot_append(
+            self._ptr(f, torch.float32, "f"), int(ld), int(q_off), int(k_off), int(v_off), self._ptr(q_out, dt, "q_out"),
+            self._ptr(q_scale, torch.float32, "q_scale"), self._ptr(k_cache, dt, "k_cache"), self._ptr(v_cache, dt, "v_cache"),
+            self._ptr(k_pool, dt, "k_pool"), self._ptr(v_pool, dt, "v_pool"), self._ptr(freq, torch.float32, "freq"), float(amp),
+            int(rot_dims), self._ptr(vfreq, torch.float32, "vfreq"), int(v_rot), int(interleaved),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+            self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._dense_code(dt),
+            int(rows), int(heads), int(kv_heads), int(dim), int(vdim), self._stream(k_cache)))
+
+    def window_attn(self, q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg: int, gate_off: int, vfreq, v_rot: bool, interleaved: bool,
+                    row_seq, row_pos, block_table, page: int, pool: int, out, rows: int, heads: int, kv_heads: int, dim: int, vdim: int,
+                    window: int) -> None:
+        dt = k_cache.dtype
+        gp = None if gate is None else self._ptr(gate, torch.float32, "gate") + gate_off * 4
+        self.lib.check(self.lib.exl2_window_attn(
+            self._ptr(q, dt, "q"), self._ptr(k_cache, dt, "k_cache"), self._ptr(v_cache, dt, "v_cache"), self._ptr(k_pool, dt, "k_pool"),
+            self._ptr(v_pool, dt, "v_pool"), self._ptr(sink, torch.float32, "sink"), gp, int(ldg), self._ptr(vfreq, torch.float32, "vfreq"),
+            int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+            self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, dt, "out"),
+            self._dense_code(dt), int(rows), int(heads), int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
 
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))

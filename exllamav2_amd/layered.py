@@ -1,5 +1,9 @@
 """Config-driven decoder stack over unquantized weights: each layer is a mixer and an optional feed-forward taken from two
-registries, joined by post-norm residual steps  x <- norm(alpha x + sublayer(x)) (1 + w)  on an fp32 residual stream.
+registries, on an fp32 residual stream.  The residual style is the configuration's: post-norm steps
+x <- norm(alpha x + sublayer(x)) (1 + w)  (RMS norm, a `head` matrix), or pre-norm steps  x <- x + sublayer(layer_norm(x))  (weight and
+bias, logits from the embedding table, optional soft cap).  Mixers: latent attention, windowed attention with pooled blocks,
+state-space scan; a stack may mix them -- each keeps what it needs between steps (pages of keys and values, per-slot recurrent
+state) under one page pool.
 
 The model has ONE forward, `step(batch, cache)`: the rows of a step are a flat list of tokens, each with its sequence slot and
 position, so whole prompts, portions of prompts and single decoded tokens of several requests run through the same launches
@@ -11,14 +15,16 @@ from dataclasses import dataclass
 
 import torch
 
-from .cache import LatentCache, PagePool
+from .cache import LatentCache, LayerStates, PagePool
 from .config import LayeredConfig
 from .dense_linear import DenseLinear
 from .ext import ext_c
 from .latent_attn import LatentAttention
-from .mlp import DenseGatedMLP
+from .mlp import DenseActMLP, DenseGatedMLP
 from .moe_mlp import ScoredMoEMLP
-from .rmsnorm import PostNorm
+from .rmsnorm import PostNorm, PreLayerNorm
+from .ssm import StateSpaceMixer
+from .window_attn import WindowAttention
 
 
 def _latent_attention(model, key, idx, spec):
@@ -29,7 +35,24 @@ def _latent_attention(model, key, idx, spec):
                            kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None))
 
 
+def _window_attention(model, key, idx, spec):
+    m = spec["mixer"]
+    mask, rot = m.get("mask") or {}, m.get("rot") or {}
+    return WindowAttention(model, key, idx, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]),
+                           vdim=int(m.get("vdim") or m["dim"]), window=int(mask.get("size") or (1 << 30)), pool=int(mask.get("pool") or 0),
+                           rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)), rot_scaling=rot.get("scaling"),
+                           scale=float(m["scale"]))
+
+
+def _state_space(model, key, idx, spec):
+    m = spec["mixer"]
+    return StateSpaceMixer(model, key, idx, heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]),
+                           groups=int(m.get("groups", 1)), norm_groups=int(m.get("norm_groups", 1)), taps=int(m["conv"]))
+
+
 def _dense_mlp(model, key, idx, spec):
+    if model.config.residual == "pre_ln":                      # two matrices, squared relu between them
+        return DenseActMLP(model, key, idx)
     return DenseGatedMLP(model, key, idx)
 
 
@@ -39,7 +62,8 @@ def _moe_mlp(model, key, idx, spec):
                         route_scale=float(r["scale"]), ff=int(e["ff"]), limit=float(e["limit"]))
 
 
-MIXERS = {"latent_attention": _latent_attention}             # config `type` -> builder(model, key, layer index, layer spec)
+# config `type` -> builder(model, key, layer index, layer spec)
+MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention, "mamba2": _state_space}
 FEED_FORWARDS = {"dense": _dense_mlp, "moe": _moe_mlp}       # config `mlp.kind` -> builder(model, key, layer index, mlp spec)
 
 
@@ -58,6 +82,9 @@ class StepBatch:
     # (row0 int32 [n], rows int32 [n], n) and single decoded tokens (row0 int32 [n], n, largest position among them)
     tiles16: tuple | None = None
     tiles1: tuple | None = None
+    # the runs of consecutive rows that one sequence brings (recurrent mixers walk them in order): (first row int32 [n],
+    # rows int32 [n], n, longest run)
+    spans_dev: tuple | None = None
     # host-side view of the same rows, one tuple per request in the step: (first row, rows, sequence slot, first position)
     spans: list | None = None
 
@@ -105,21 +132,28 @@ class LayeredModel:
         self.embed = need("embed")
         if tuple(self.embed.shape) != (cfg.vocab, cfg.width):
             raise RuntimeError(f"embed is {tuple(self.embed.shape)}, config says {(cfg.vocab, cfg.width)}")
+        pre = cfg.residual == "pre_ln"
+
+        def make_norm(name):
+            if pre:
+                return PreLayerNorm(self.ext, name, need(name), need(name + ".b") if name + ".b" in tensors else None, cfg.norm_eps)
+            return PostNorm(self.ext, name, need(name), cfg.norm_eps, cfg.postln_alpha)
+
         self.layers = []
         for i, spec in enumerate(cfg.layers):
             key = f"l{i}"
             if spec["type"] not in MIXERS:
                 raise RuntimeError(f"layer {i}: unknown mixer type '{spec['type']}' (known: {sorted(MIXERS)})")
             mixer = MIXERS[spec["type"]](self, key, i, spec).load(lambda n, k=key: need(f"{k}.mix.{n}"))
-            norm1 = PostNorm(self.ext, key + ".norm1", need(key + ".norm1"), cfg.norm_eps, cfg.postln_alpha)
+            norm1 = make_norm(key + ".norm1")
             ff, norm2 = None, None
             ms = spec.get("mlp")
             if ms is not None:
                 if ms["kind"] not in FEED_FORWARDS:
                     raise RuntimeError(f"layer {i}: unknown feed-forward kind '{ms['kind']}' (known: {sorted(FEED_FORWARDS)})")
                 ff = FEED_FORWARDS[ms["kind"]](self, key + ".mlp", i, ms).load(lambda n, k=key: need(f"{k}.mlp.{n}"))
-            if ff is not None or key + ".norm2" in tensors:
-                norm2 = PostNorm(self.ext, key + ".norm2", need(key + ".norm2"), cfg.norm_eps, cfg.postln_alpha)
+            if ff is not None or (not pre and key + ".norm2" in tensors):
+                norm2 = make_norm(key + ".norm2")
             self.layers.append((mixer, norm1, ff, norm2))
         for i, (mixer, *_rest) in enumerate(self.layers):
             j = getattr(mixer, "kv_from", None)
@@ -129,12 +163,22 @@ class LayeredModel:
                 src = self.layers[j][0]
                 if (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
                     raise RuntimeError(f"layer {i}: its latent sizes / rotation differ from layer {j}'s, whose cache it reads")
-        self.final_norm = need("final.norm")
-        self.head = DenseLinear(self.ext, "head", need("head"))
+        if pre:
+            self.final_norm = make_norm("final.norm")
+            # the sublayers in order, each with the norm in front of it: (norm, module, is a mixer)
+            self.sublayers = []
+            for mixer, norm1, ff, norm2 in self.layers:
+                self.sublayers.append((norm1, mixer, True))
+                if ff is not None:
+                    self.sublayers.append((norm2, ff, False))
+        else:
+            self.final_norm = need("final.norm")
+        self.head = DenseLinear(self.ext, "head", self.embed if cfg.tied_head else need("head"))
         self.loaded = True
         return self
 
     def weight_bytes(self) -> int:
+        """bytes a decoded token streams (a tied output table counts once: the embedding reads one row of it)"""
         n = self.head.weight_bytes()
         for mixer, _n1, ff, _n2 in self.layers:
             n += mixer.weight_bytes() + (ff.weight_bytes() if ff is not None else 0)
@@ -142,7 +186,9 @@ class LayeredModel:
 
     # ---- cache ----------------------------------------------------------------------------------------------------------------
 
-    def make_cache(self, pool: PagePool) -> LatentCache:
+    def make_cache(self, pool: PagePool):
+        if any(hasattr(mixer, "make_state") for mixer, *_rest in self.layers):
+            return LayerStates(pool, {i: mixer.make_state(pool, self.dtype) for i, (mixer, *_rest) in enumerate(self.layers)})
         widths, owner = {}, {}
         for i, (mixer, *_rest) in enumerate(self.layers):
             if mixer.kv_from is None:
@@ -158,6 +204,8 @@ class LayeredModel:
         """Runs the batch's rows through all layers, appending to the cache; returns fp32 logits [n_logits, vocab] (None if
         no row wants them)."""
         ext, cfg, rows = self.ext, self.config, batch.rows
+        if cfg.residual == "pre_ln":
+            return self._step_pre_norm(batch, cache)
         x32 = self.buf("x32", (rows, self.width), torch.float32)
         xh = x32 if self.dtype is torch.float32 else self.buf("xh", (rows, self.width), self.dtype)
         ext.embed_scale(self.embed, batch.ids, x32, xh, cfg.embedding_scale)
@@ -176,3 +224,24 @@ class LayeredModel:
         ext.rms_rows(x32, self.width, self.final_norm, True, xn, self.width, batch.n_logits, self.width, cfg.norm_eps,
                      row_idx=batch.logit_rows)
         return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), torch.float32))
+
+    def _step_pre_norm(self, batch: StepBatch, cache) -> torch.Tensor | None:
+        """x <- x + sublayer(layer_norm(x)): every residual addition runs in ONE launch with the layer norm of the sublayer that
+        follows it; the last addition stands alone and the final norm is taken of the rows whose logits are wanted only."""
+        ext, cfg, rows = self.ext, self.config, batch.rows
+        x32 = self.buf("x32", (rows, self.width), torch.float32)
+        xh = self.buf("xh", (rows, self.width), self.dtype)
+        ext.embed_scale(self.embed, batch.ids, x32, None, cfg.embedding_scale)
+        y = None
+        for norm, module, is_mixer in self.sublayers:
+            norm.forward(x32, y, xh, rows)
+            y = module.forward(xh, rows, batch, cache) if is_mixer else module.forward(xh, rows)[0]
+        if y is not None:
+            ext.add_layer_norm(x32, y, None, None, None, rows, cfg.norm_eps)
+        if batch.n_logits == 0:
+            return None
+        xn = self.buf("xn", (batch.n_logits, self.width), self.dtype)
+        self.final_norm.forward(x32, None, xn, batch.n_logits, row_idx=batch.logit_rows)
+        cap = cfg.logit_softcap
+        return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), torch.float32),
+                                 epi=ext.EPI_SOFT_CAP if cap > 0 else ext.EPI_NONE, limit=cap)

@@ -64,3 +64,28 @@ class DenseGatedMLP:
         g = self.gate.forward(xh, rows, out=m.buf("ff.g", (rows, ff), torch.float32))
         a = self.up.forward(xh, rows, out=m.buf("ff.a", (rows, ff), m.dtype), aux=g, aux_ld=ff, epi=self.ext.EPI_SILU_AUX_MUL)
         return self.down.forward(a, rows, out=m.buf("ff.y", (rows, m.width), torch.float32)), None
+
+
+class DenseActMLP:
+    """Two-matrix feed-forward over unquantized weights: W_down act(W_up h), the activation in the up projection's epilogue
+    (csrc/dense.hip).  act: an epilogue code of the dense linear (default relu(z)^2)."""
+
+    def __init__(self, model, key: str, layer_idx: int, act: int | None = None):
+        self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
+        self.act = self.ext.EPI_RELU_SQUARED if act is None else act
+
+    def load(self, get):
+        from .dense_linear import DenseLinear
+        self.up = DenseLinear(self.ext, self.key + ".up", get("up"))
+        self.down = DenseLinear(self.ext, self.key + ".down", get("down"))
+        if self.down.in_features != self.up.out_features:
+            raise RuntimeError(f"{self.key}: up is {tuple(self.up.weight.shape)}, down is {tuple(self.down.weight.shape)}")
+        return self
+
+    def weight_bytes(self) -> int:
+        return self.up.weight_bytes() + self.down.weight_bytes()
+
+    def forward(self, xh: torch.Tensor, rows: int):
+        m, ff = self.model, self.up.out_features
+        a = self.up.forward(xh, rows, out=m.buf("ff.a", (rows, ff), m.dtype), epi=self.act)
+        return self.down.forward(a, rows, out=m.buf("ff.y", (rows, m.width), torch.float32)), None

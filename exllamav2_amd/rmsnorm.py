@@ -36,3 +36,18 @@ class PostNorm:
 
     def forward(self, x32: torch.Tensor, xh, y, rows: int, moe=None) -> None:
         self.ext.post_norm(x32, xh, y, self.weight, rows, self.alpha, self.eps, moe=moe)
+
+
+class PreLayerNorm:
+    """The norm in front of a sublayer of a pre-norm layer: (x - mean) / sqrt(var + eps) * w + b.  It runs fused with the residual
+    addition of the sublayer BEFORE it (csrc/rowops.hip: add_layer_norm_kernel): `forward` adds `y` (that sublayer's fp32 output, or
+    None at the start of the stack) into the fp32 stream and leaves the normalised rows in the operand dtype."""
+
+    def __init__(self, ext, key: str, weight: torch.Tensor, bias: torch.Tensor | None, eps: float):
+        self.ext, self.key, self.weight, self.eps = ext, key, weight.contiguous(), eps
+        self.bias = bias.contiguous() if bias is not None else None
+        if self.bias is not None and self.bias.shape != self.weight.shape:
+            raise RuntimeError(f"{key}: weight and bias differ in shape")
+
+    def forward(self, x32: torch.Tensor, y, out: torch.Tensor, rows: int, row_idx=None) -> None:
+        self.ext.add_layer_norm(x32, y, self.weight, self.bias, out, rows, self.eps, row_idx=row_idx)

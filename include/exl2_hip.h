@@ -436,6 +436,61 @@ int exl2_latent_attn_tiles(const void* q, int ldq, int q_head_stride, int q_rot_
                            int nsplit, int heads, int kv_rank, int rot, int rot_dims, const float* inv_freq, float scale,
                            int window, void* stream);
 
+/* exl2_dense_linear with a bias: bias fp32 [N] (nullable) is added to the accumulator before the epilogue; plain one-slab calls
+   only.  Further epilogues: 4 relu(acc)^2, 5 the soft cap limit * tanh(acc / limit). */
+int exl2_dense_linear_bias(const void* x, const void* w, const float* bias, void* y, const float* aux, int dtype, int y_f32,
+                           int M, int N, int K, int ldx, int ldw, int ldy, int ldaux,
+                           int batch, long long sxb, long long swb, long long syb, long long sauxb,
+                           const int* w_sel, int n_sel, const int* grp_count, const int* grp_offset, const int* grp_rows,
+                           int x_div, int epi, float limit, void* stream);
+/* the pre-norm residual step: x[r] += y[r] (y nullable) on the fp32 stream, then out[r] = (x - mean) / sqrt(var + eps) * w + b in
+   the operand dtype (or fp32); w == NULL: only the addition.  row_idx (nullable, no addition then): output row r is made from
+   stream row row_idx[r]. */
+int exl2_add_layer_norm(float* x, const float* y, const void* w, const void* b, void* out, int out_f32, const int* row_idx,
+                        int dtype, int rows, int width, float eps, void* stream);
+
+/* ---- state-space mixer (csrc/ssm.hip).  A span is the run of consecutive rows one sequence brings to the step: span i = rows
+   span_row0[i] .. + span_rows[i]; its slot and first position are row_seq / row_pos of its first row.  A span at position 0
+   starts from zeros whatever its slot holds. */
+
+/* out[r, c] = silu(bias[c] + sum_k w[c, k] in(pos - (taps - 1) + k)[c]) per channel over the sequence's own earlier inputs (this
+   span's rows, then tail [slots, taps - 1, channels], zeros before the sequence's start); afterwards the tails hold the last
+   taps - 1 inputs of every span's sequence.  w [channels, taps] / bias [channels] in the operand dtype; in / out fp32. */
+int exl2_conv_silu_rows(const float* in, int ld, const void* w, const void* bias, float* out, int ldo, float* tail,
+                        const int* span_row0, const int* span_rows, int spans, int max_span_rows, const int* row_seq,
+                        const int* row_pos, int dtype, int channels, int taps, void* stream);
+/* per head h (group h / (heads / groups)) and row: d = softplus(dt + dt_bias[h]); S <- exp(-exp(A_log[h]) d) S + d B u^T;
+   y = S^T C + D[h] u.  u [rows, ldu] head h at h * vdim; B, C [rows, ldbc] group g at g * n_state; dt [rows, lddt]; state fp32
+   [slots, heads, n_state, vdim], read at a span's start (unless it starts at position 0) and written at its end. */
+int exl2_ssm_scan(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
+                  const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
+                  const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
+                  int heads, int groups, int n_state, int vdim, void* stream);
+/* out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part] for each of `groups` equal parts of the dim values */
+int exl2_gated_group_norm(const float* y, int ldy, const float* z, int ldz, const void* w, void* out, int ldo, int out_f32,
+                          int dtype, int rows, int dim, int groups, float eps, void* stream);
+
+/* ---- windowed attention with pooled blocks, a sink and rotated values (csrc/window_attn.hip).  Cache: keys [pages, page,
+   kv_heads, dim], values [pages, page, kv_heads, vdim]; pooled rows [pages, ceil(page / pool), kv_heads, dim | vdim] (block b
+   of `pool` tokens at index ((b pool) % page) / pool of its first token's page). */
+
+/* new rows from the projection output f fp32 [rows, ld] (q at q_off, k at k_off, v at v_off): q and k rotated over their first
+   rot_dims values by pos * freq[i] (cos and sin times amp; pairs in halves or interleaved), v over all vdim values by
+   pos * vfreq[m] when v_rot; q times q_scale[head] to q_out [rows, heads, dim]; k and v into the cache at (row_seq, row_pos); then
+   every row whose position completes a block of `pool` tokens writes the block's mean key and mean value (pool 0: none). */
+int exl2_kv_rot_append(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
+                       void* k_cache, void* v_cache, void* k_pool, void* v_pool, const float* freq, float amp, int rot_dims,
+                       const float* vfreq, int v_rot, int interleaved, const int* row_seq, const int* row_pos,
+                       const int* block_table, int bt_stride, int page, int pool, int dtype, int rows, int heads,
+                       int kv_heads, int dim, int vdim, void* stream);
+/* out[r, h] = turn_back(sum_j p_j v_j, pos) * sigmoid(gate[r, h]) over the tokens 0 <= pos - j < window and the pooled blocks
+   wholly in front of the window; p_j = exp(q . k_j) / (exp(sink[h]) + sum exp(q . k)) (sink nullable).  q [rows, heads, dim] as
+   exl2_kv_rot_append left it; gate fp32 [rows, ldg] (nullable); out [rows, heads, vdim] operand dtype. */
+int exl2_window_attn(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                     const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                     const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                     void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
