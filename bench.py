@@ -61,11 +61,13 @@ def parse():
     p.add_argument("--windows", type=int, default=5, help="timed windows of --steps steps (each after --warmup untimed steps from the same "
                                                            "cache position); the MEDIAN window is the reported value")
     p.add_argument("--headline-only", action="store_true", help="= --no-cpu-baseline --no-prefill --no-dropin --no-ctx-window (A/B runs)")
-    p.add_argument("--design", default=None, choices=["benolix"],
-                   help="instead of the headline: prefill / decode throughput of the latent-attention layer stack at real layer sizes "
-                        "beside the quantized Mixtral-style stack of equal size (exllamav2_amd/bench_layered.py); one JSON line each")
+    p.add_argument("--design", default=None, choices=["benolix", "tibalorn"],
+                   help="instead of the headline: prefill / decode throughput of a layer-stack design at real layer sizes beside the "
+                        "package's closest other model of equal size (benolix: latent attention + MoE beside the quantized Mixtral-style "
+                        "stack; tibalorn: state-space + windowed attention beside a latent-attention stack; "
+                        "exllamav2_amd/bench_layered.py); one JSON line each")
     p.add_argument("--design-sizes", default="w2048,w4096")
-    p.add_argument("--design-no-peer", action="store_true", help="--design: skip the quantized peer model")
+    p.add_argument("--design-no-peer", action="store_true", help="--design: skip the peer model")
     a = p.parse_args()
     if a.headline_only:
         a.no_cpu_baseline = a.no_prefill = a.no_dropin = a.no_ctx_window = True
@@ -754,7 +756,7 @@ def main():
     if "--design" in sys.argv:
         a = parse()
         from exllamav2_amd import bench_layered
-        bench_layered.run(a.design_sizes.split(","), peer=not a.design_no_peer)
+        bench_layered.run(a.design_sizes.split(","), peer=not a.design_no_peer, design=a.design)
         return
     args = parse()
     if args.cpu_baseline_only:

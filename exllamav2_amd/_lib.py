@@ -120,9 +120,13 @@ PROTOTYPES = {
     # state-space mixer (csrc/ssm.hip), windowed attention with pooled blocks (csrc/window_attn.hip)
     "exl2_conv_silu_rows": (ci, [vp, ci, vp, vp, vp, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, vp]),
     "exl2_ssm_scan": (ci, [vp, ci, vp, vp, ci, vp, ci, vp, vp, vp, vp, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, ci, vp]),
+    "exl2_ssm_scan_chunked_supported": (ci, [ci, ci]),
+    "exl2_ssm_scan_chunked": (ci, [vp, ci, vp, vp, ci, vp, ci, vp, vp, vp, vp, ci, vp, vp, vp, vp, ci, ci, ci, vp, vp, vp, vp, ci, ci, ci, ci, vp]),
     "exl2_gated_group_norm": (ci, [vp, ci, vp, ci, vp, vp, ci, ci, ci, ci, ci, ci, cf, vp]),
     "exl2_kv_rot_append": (ci, [vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, vp, cf, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]),
     "exl2_window_attn": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
+    "exl2_window_attn_tiles_supported": (ci, [ci, ci]),
+    "exl2_window_attn_tiles": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

@@ -1,6 +1,7 @@
-"""Prefill and decode throughput of a latent-attention / scored-MoE layer stack at layer sizes of real models (random weights),
-beside the closest quantized model of the package (a Mixtral-style EXL2 stack) at the same width, expert width, expert count and
-depth.  Used by `bench.py --design benolix`; one JSON object per size."""
+"""Prefill and decode throughput of the layer-stack models at layer sizes of real models (random weights), each beside the closest
+other model of the package at equal size: the latent-attention / scored-MoE stack beside a Mixtral-style EXL2 stack (same width,
+expert width, expert count, depth), the state-space / windowed-attention stack beside a latent-attention stack (same width, depth,
+heads, window, feed-forward parameters).  Used by `bench.py --design benolix | tibalorn`; one JSON object per size and model."""
 from __future__ import annotations
 
 import json
@@ -56,6 +57,8 @@ def random_tensors(cfg: dict, device, seed: int = 0) -> dict:
             mat(k + ".mix.dkv", R + rd, w); vec(k + ".mix.dkv.norm", R, 1.0)
         mat(k + ".mix.uk", H * dim, R); mat(k + ".mix.uv", H * vd, R); mat(k + ".mix.g", H * vd, w); mat(k + ".mix.o", w, H * vd)
         ms = L["mlp"]
+        if ms is None:
+            continue
         if ms["kind"] == "dense":
             mat(k + ".mlp.gate", ms["ff"], w); mat(k + ".mlp.up", ms["ff"], w); mat(k + ".mlp.down", w, ms["ff"])
         else:
@@ -153,8 +156,130 @@ def bench_quantized_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: in
     return out
 
 
-def run(sizes, device="cuda:0", peer: bool = True):
+# ---- pre-norm stacks of state-space and windowed-attention mixers (Tibalorn) -----------------------------------------------------
+
+HYBRID_SIZES = {
+    # a 3 : 1 pattern of state-space and attention layers; state-space inner width = 2 x width in heads of 64, state 128; attention
+    # with grouped heads of 128, a window of 1024 and pooled blocks of 64 behind it; squared-relu feed-forward behind the attention
+    "w2048": dict(width=2048, ssm_heads=64, ssm_vdim=64, state=128, groups=1, norm_groups=1, taps=4, heads=16, kv_heads=4, dim=128,
+                  vdim=128, window=1024, pool=64, rot_dims=64, ff=8192, pattern="ssa+s", vocab=32000),
+    "w4096": dict(width=4096, ssm_heads=128, ssm_vdim=64, state=128, groups=8, norm_groups=8, taps=4, heads=32, kv_heads=8, dim=128,
+                  vdim=128, window=2048, pool=64, rot_dims=128, ff=14336, pattern="sa+", vocab=32000),
+}
+
+
+def hybrid_config(s: dict) -> dict:
+    """pattern: s = state-space layer, a = attention layer, + = the layer before it has a feed-forward"""
+    layers = []
+    for ch in s["pattern"]:
+        if ch == "+":
+            layers[-1]["mlp"] = {"ff": s["ff"], "kind": "dense"}
+        elif ch == "s":
+            layers.append({"type": "mamba2", "mlp": None,
+                           "mixer": {"conv": s["taps"], "groups": s["groups"], "heads": s["ssm_heads"], "norm_groups": s["norm_groups"],
+                                     "state": s["state"], "vdim": s["ssm_vdim"]}})
+        else:
+            layers.append({"type": "attention", "mlp": None,
+                           "mixer": {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"],
+                                     "mask": {"pool": s["pool"], "size": s["window"]}, "scale": s["dim"] ** -0.5,
+                                     "rot": {"base": 1e6, "dims": s["rot_dims"],
+                                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}})
+    return {"architecture": "Tibalorn", "embedding": {"scale": 1.0}, "layers": layers, "logit_softcap": 30.0, "norm": {"eps": 1e-5},
+            "vocab": s["vocab"], "width": s["width"]}
+
+
+def hybrid_random_tensors(cfg: dict, device, seed: int = 0) -> dict:
+    g = torch.Generator(device=device).manual_seed(seed)
+    T = {}
+
+    def mat(name, out, inp, gain=1.0):
+        T[name] = (torch.randn((out, inp), device=device, generator=g) * gain / inp ** 0.5).to(torch.bfloat16)
+
+    def vec(name, n, centre, spread=0.1):
+        T[name] = (centre + spread * torch.randn((n,), device=device, generator=g)).to(torch.bfloat16)
+
+    w = cfg["width"]
+    T["embed"] = (torch.randn((cfg["vocab"], w), device=device, generator=g) * 0.5).to(torch.bfloat16)
+    vec("final.norm", w, 1.0); vec("final.norm.b", w, 0.0)
+    for i, L in enumerate(cfg["layers"]):
+        m, k = L["mixer"], f"l{i}"
+        vec(k + ".norm1", w, 1.0); vec(k + ".norm1.b", w, 0.0)
+        if L["type"] == "mamba2":
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            mat(k + ".mix.in", 2 * inner + 2 * gn + m["heads"], w); mat(k + ".mix.conv", inner + 2 * gn, m["conv"])
+            vec(k + ".mix.conv.b", inner + 2 * gn, 0.0); vec(k + ".mix.dt_bias", m["heads"], -1.0, 0.5); vec(k + ".mix.A_log", m["heads"], 0.0, 0.5)
+            vec(k + ".mix.D", m["heads"], 1.0); vec(k + ".mix.norm", inner, 1.0); mat(k + ".mix.o", w, inner)
+        else:
+            H, G, dim, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", H * dim, w); mat(k + ".mix.k", G * dim, w); mat(k + ".mix.v", G * vd, w); mat(k + ".mix.g", H * vd, w)
+            vec(k + ".mix.q.b", H * dim, 0.0); vec(k + ".mix.k.b", G * dim, 0.0); vec(k + ".mix.v.b", G * vd, 0.0)
+            vec(k + ".mix.temp", H, 1.0); vec(k + ".mix.sink", H, 0.0, 1.0); mat(k + ".mix.o", w, H * vd)
+        if L["mlp"] is not None:
+            vec(k + ".norm2", w, 1.0); vec(k + ".norm2.b", w, 0.0)
+            mat(k + ".mlp.up", L["mlp"]["ff"], w); mat(k + ".mlp.down", w, L["mlp"]["ff"])
+    return T
+
+
+def _bench_engine(model, out, vocab, prompt, ctx, decode_steps, batches):
+    from .engine import Engine
+    g = torch.Generator().manual_seed(1)
+    toks = torch.randint(0, vocab, (prompt,), generator=g).tolist()
+    eng = Engine(model, max_tokens=max(prompt, max(batches) * (ctx + decode_steps + 8)) + 256, max_seqs=max(4, max(batches)))
+    eng.step([("warm", toks, [prompt - 1])], ["warm"])
+    dt = _timed(lambda: eng.step([("p", toks, [prompt - 1])], ["p"]), 3)
+    out["prefill_tokens_per_s"] = prompt / dt
+    out["prefill_ms"] = dt * 1e3
+    for b in batches:
+        ids = [f"d{i}" for i in range(b)]
+        eng.step([(r, toks[:ctx], []) for r in ids])
+        step = lambda: eng.step([(r, [7], [0]) for r in ids])
+        step()
+        dt = _timed(step, decode_steps)
+        out[f"decode_b{b}_tokens_per_s"] = b / dt
+        out[f"decode_b{b}_ms_per_step"] = dt * 1e3
+        for r in ids:
+            eng.finish(r)
+    eng.close()
+    return out
+
+
+def bench_hybrid(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = HYBRID_SIZES[size]
+    cfg = hybrid_config(s)
+    model = LayeredModel(LayeredConfig.from_dict_prenorm(cfg), device=device, dtype=torch.bfloat16).load(hybrid_random_tensors(cfg, device))
+    out = {"design": "tibalorn", "size": size, "layers": len(cfg["layers"]), "pattern": s["pattern"], "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
+def bench_hybrid_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    """the closest model of the package: a latent-attention stack (bfloat16, the same engine) of the same width, depth, head count,
+    window and vocabulary, with dense feed-forwards of the same width behind the same layers"""
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = HYBRID_SIZES[size]
+    hyb = hybrid_config(s)
+    layers = []
+    for L in hyb["layers"]:
+        mixer = {"dim": s["dim"], "heads": s["heads"], "kv_rank": 512, "mask": {"size": s["window"]}, "q_rank": s["width"] * 3 // 8,
+                 "rot": {"base": 10000.0, "dims": 64}, "rot_dim": 64, "scale": (s["dim"] + 64) ** -0.5, "vdim": s["vdim"]}
+        layers.append({"type": "latent_attention", "mixer": mixer,
+                       "mlp": {"ff": s["ff"] * 2 // 3 // 64 * 64, "kind": "dense"} if L["mlp"] is not None else None})
+    cfg = {"architecture": "Benolix", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5}, "postln_alpha": 1.0,
+           "vocab": s["vocab"], "width": s["width"]}
+    model = LayeredModel(LayeredConfig.from_dict(cfg), device=device, dtype=torch.bfloat16).load(random_tensors(cfg, device))
+    out = {"design": "benolix-dense-peer", "size": size, "layers": len(layers), "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
+def run(sizes, device="cuda:0", peer: bool = True, design: str = "benolix"):
     for size in sizes:
+        if design == "tibalorn":
+            print(json.dumps(bench_hybrid(size, device)), flush=True)
+            if peer:
+                print(json.dumps(bench_hybrid_peer(size, device)), flush=True)
+            continue
         print(json.dumps(bench_layered(size, device)), flush=True)
         if peer:
             print(json.dumps(bench_quantized_peer(size, device)), flush=True)

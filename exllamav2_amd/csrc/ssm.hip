@@ -10,6 +10,7 @@
 // All arithmetic is fp32; inputs are the fp32 outputs of the mixer's input projection.
 #include "hw.h"
 #include "errors.h"
+#include <stdint.h>
 
 template <typename T> DEV float ss_ld(const T* p);
 template <> DEV float ss_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
@@ -210,6 +211,235 @@ KERNEL void __launch_bounds__(256) scan_kernel(const ScanArgs a)
     }
 }
 
+// ---- the same scan in chunks (portions of prompts) ----------------------------------------------------------------------------------
+// Inside a chunk of SSD_L tokens the recurrence unrolls into small matrix products (all fp32 FMA, 4 x 4 register tiles over LDS):
+// with l_t = the log decay of token t, c_t = l_1 + .. + l_t, x_t = d_t u_t,
+//     y_t = exp(c_t) S_in^T C_t + sum_{s <= t} exp(c_t - c_s) (C_t . B_s) x_s + D u_t,      S_out = exp(c_L) S_in + sum_s exp(c_L - c_s) B_s x_s^T.
+// Three launches make every (chunk, head) of a step independent work: (1) each chunk's own contribution Z to S_out and its total
+// decay, (2) the carry over a span's chunks, one thread per state element (Z is replaced by the state ENTERING the chunk, the slot
+// takes the state after the last), (3) each chunk's outputs.  Every exponent is <= 0.
+
+#define SSD_L 64
+
+struct SsdArgs
+{
+    ScanArgs s;
+    float* zbuf;                             // [chunks of the step, heads, N, P]
+    float* dbuf;                             // [chunks of the step, heads]: exp(c_L)
+    const int* span_chunk0;                  // first chunk of every span
+};
+
+// step sizes, log decays and their running sum for the chunk's tokens (rows past the chunk's end: zeros); thread t < SSD_L = token t
+DEV void ssd_stage_decay(const ScanArgs& a, int h, long long row0, int lc, float* s_dt, float* s_cum)
+{
+    const int t = tid();
+    if (t < SSD_L)
+    {
+        float d = 0.0f;
+        if (t < lc) d = ss_softplus(a.dt[(row0 + t) * a.lddt + h] + a.dt_bias[h]);
+        s_dt[t] = d;
+        s_cum[t] = -expf(a.A_log[h]) * d;
+    }
+    block_sync();
+    if (t == 0)
+    {
+        float c = 0.0f;
+        for (int i = 0; i < SSD_L; i++) { c += s_cum[i]; s_cum[i] = c; }
+    }
+    block_sync();
+}
+
+KERNEL void __launch_bounds__(256) ssd_chunk_state_kernel(const SsdArgs g)
+{
+    DYN_SMEM(smem);
+    const ScanArgs& a = g.s;
+    const int c = bid_x(), h = bid_y(), sp = bid_z();
+    const int n_tok = a.span_rows[sp];
+    if (c * SSD_L >= n_tok) return;
+    const long long row0 = a.span_row0[sp] + c * SSD_L;
+    const int lc = min(SSD_L, n_tok - c * SSD_L);
+    const int N = a.N, P = a.P, grp = h / (a.heads / a.groups), t = tid();
+    float* s_dt = (float*)smem;                                  // [L]
+    float* s_cum = s_dt + SSD_L;                                 // [L]
+    float* s_B = s_cum + SSD_L;                                  // [L][N]: B_s exp(c_L - c_s)
+    float* s_X = s_B + SSD_L * N;                                // [L][P]: d_s u_s
+    ssd_stage_decay(a, h, row0, lc, s_dt, s_cum);
+    const float c_end = s_cum[SSD_L - 1];
+    for (int i = t; i < SSD_L * N; i += 256)
+    {
+        const int tok = i / N, n = i % N;
+        s_B[i] = tok < lc ? a.B[(row0 + tok) * a.ldbc + grp * N + n] * expf(c_end - s_cum[tok]) : 0.0f;
+    }
+    for (int i = t; i < SSD_L * P; i += 256)
+    {
+        const int tok = i / P, p = i % P;
+        s_X[i] = tok < lc ? a.u[(row0 + tok) * a.ldu + h * P + p] * s_dt[tok] : 0.0f;
+    }
+    block_sync();
+    float* z = g.zbuf + ((long long)(g.span_chunk0[sp] + c) * a.heads + h) * (long long)N * P;
+    const int tp = P / 4, tiles = (N / 4) * tp;
+    for (int tile = t; tile < tiles; tile += 256)
+    {
+        const int n0 = (tile / tp) * 4, p0 = (tile % tp) * 4;
+        float acc[4][4] = {};
+        for (int k = 0; k < SSD_L; k++)
+        {
+            const f32x4 b = *(const f32x4*)(s_B + k * N + n0), x = *(const f32x4*)(s_X + k * P + p0);
+            #pragma unroll
+            for (int i = 0; i < 4; i++)
+                #pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(b[i], x[j], acc[i][j]);
+        }
+        #pragma unroll
+        for (int i = 0; i < 4; i++) *(f32x4*)(z + (long long)(n0 + i) * P + p0) = (f32x4){acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+    }
+    if (t == 0) g.dbuf[(long long)(g.span_chunk0[sp] + c) * a.heads + h] = expf(c_end);
+}
+
+// grid (ceil(N P / 256), heads, spans)
+KERNEL void __launch_bounds__(256) ssd_carry_kernel(const SsdArgs g)
+{
+    const ScanArgs& a = g.s;
+    const int e = bid_x() * 256 + tid(), h = bid_y(), sp = bid_z();
+    const long long NP = (long long)a.N * a.P;
+    if (e >= NP) return;
+    const int r0 = a.span_row0[sp];
+    const int chunks = (a.span_rows[sp] + SSD_L - 1) / SSD_L;
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * NP + e;
+    float S = a.row_pos[r0] > 0 ? *st : 0.0f;
+    const long long c0 = g.span_chunk0[sp];
+    int c = 0;
+    for (; c + 4 <= chunks; c += 4)                              // the loads of four chunks leave together, the chain follows
+    {
+        float zv[4], dv[4];
+        #pragma unroll
+        for (int i = 0; i < 4; i++)
+        {
+            zv[i] = g.zbuf[((c0 + c + i) * a.heads + h) * NP + e];
+            dv[i] = g.dbuf[(c0 + c + i) * a.heads + h];
+        }
+        #pragma unroll
+        for (int i = 0; i < 4; i++)
+        {
+            g.zbuf[((c0 + c + i) * a.heads + h) * NP + e] = S;
+            S = fmaf(dv[i], S, zv[i]);
+        }
+    }
+    for (; c < chunks; c++)
+    {
+        const float zv = g.zbuf[((c0 + c) * a.heads + h) * NP + e], dv = g.dbuf[(c0 + c) * a.heads + h];
+        g.zbuf[((c0 + c) * a.heads + h) * NP + e] = S;
+        S = fmaf(dv, S, zv);
+    }
+    *st = S;
+}
+
+KERNEL void __launch_bounds__(256) ssd_chunk_out_kernel(const SsdArgs g)
+{
+    DYN_SMEM(smem);
+    const ScanArgs& a = g.s;
+    const int c = bid_x(), h = bid_y(), sp = bid_z();
+    const int n_tok = a.span_rows[sp];
+    if (c * SSD_L >= n_tok) return;
+    const long long row0 = a.span_row0[sp] + c * SSD_L;
+    const int lc = min(SSD_L, n_tok - c * SSD_L);
+    const int N = a.N, P = a.P, grp = h / (a.heads / a.groups), t = tid();
+    const int NS = N + 4;                                        // row stride of the [token][state] images: rows fall into different banks
+    float* s_dt = (float*)smem;                                  // [L]
+    float* s_cum = s_dt + SSD_L;                                 // [L]
+    float* s_C = s_cum + SSD_L;                                  // [L][NS]
+    float* s_BS = s_C + SSD_L * NS;                              // [L][NS] B, later [N][P] the state entering the chunk
+    float* s_X = s_BS + max(SSD_L * NS, N * P);                  // [L][P]
+    float* s_M = s_X + SSD_L * P;                                // [L][L + 4]
+    const int MS = SSD_L + 4;
+    ssd_stage_decay(a, h, row0, lc, s_dt, s_cum);
+    for (int i = t; i < SSD_L * N; i += 256)
+    {
+        const int tok = i / N, n = i % N;
+        const bool live = tok < lc;
+        s_C[tok * NS + n] = live ? a.C[(row0 + tok) * a.ldbc + grp * N + n] : 0.0f;
+        s_BS[tok * NS + n] = live ? a.B[(row0 + tok) * a.ldbc + grp * N + n] : 0.0f;
+    }
+    for (int i = t; i < SSD_L * P; i += 256)
+    {
+        const int tok = i / P, p = i % P;
+        s_X[i] = tok < lc ? a.u[(row0 + tok) * a.ldu + h * P + p] * s_dt[tok] : 0.0f;
+    }
+    block_sync();
+    // M[t][s] = (C_t . B_s) exp(c_t - c_s) for s <= t, 0 above the diagonal: one 4 x 4 tile per thread
+    {
+        const int t0 = (t / (SSD_L / 4)) * 4, s0 = (t % (SSD_L / 4)) * 4;
+        float acc[4][4] = {};
+        if (s0 <= t0 + 3)
+            for (int n = 0; n < N; n += 4)
+            {
+                f32x4 cv[4], bv[4];
+                #pragma unroll
+                for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (t0 + i) * NS + n); bv[i] = *(const f32x4*)(s_BS + (s0 + i) * NS + n); }
+                #pragma unroll
+                for (int i = 0; i < 4; i++)
+                    #pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        #pragma unroll
+                        for (int k = 0; k < 4; k++) acc[i][j] = fmaf(cv[i][k], bv[j][k], acc[i][j]);
+            }
+        #pragma unroll
+        for (int i = 0; i < 4; i++)
+            #pragma unroll
+            for (int j = 0; j < 4; j++)
+                s_M[(t0 + i) * MS + s0 + j] = s0 + j <= t0 + i ? acc[i][j] * expf(s_cum[t0 + i] - s_cum[s0 + j]) : 0.0f;
+    }
+    block_sync();                                                // B is no longer needed: its place takes the entering state
+    {
+        const float* zin = g.zbuf + ((long long)(g.span_chunk0[sp] + c) * a.heads + h) * (long long)N * P;
+        for (int i = t * 4; i < N * P; i += 1024) *(f32x4*)(s_BS + i) = *(const f32x4*)(zin + i);
+    }
+    block_sync();
+    const float Dh = a.D[h];
+    const int tp = P / 4, tiles = (SSD_L / 4) * tp;
+    for (int tile = t; tile < tiles; tile += 256)
+    {
+        const int t0 = (tile / tp) * 4, p0 = (tile % tp) * 4;
+        if (t0 >= lc) continue;
+        float inter[4][4] = {}, intra[4][4] = {};
+        for (int n = 0; n < N; n += 4)
+        {
+            f32x4 cv[4], sv[4];
+            #pragma unroll
+            for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (t0 + i) * NS + n); sv[i] = *(const f32x4*)(s_BS + (n + i) * P + p0); }
+            #pragma unroll
+            for (int i = 0; i < 4; i++)
+                #pragma unroll
+                for (int k = 0; k < 4; k++)
+                    #pragma unroll
+                    for (int j = 0; j < 4; j++) inter[i][j] = fmaf(cv[i][k], sv[k][j], inter[i][j]);
+        }
+        for (int s0 = 0; s0 <= t0; s0 += 4)
+        {
+            f32x4 mv[4], xv[4];
+            #pragma unroll
+            for (int i = 0; i < 4; i++) { mv[i] = *(const f32x4*)(s_M + (t0 + i) * MS + s0); xv[i] = *(const f32x4*)(s_X + (s0 + i) * P + p0); }
+            #pragma unroll
+            for (int i = 0; i < 4; i++)
+                #pragma unroll
+                for (int k = 0; k < 4; k++)
+                    #pragma unroll
+                    for (int j = 0; j < 4; j++) intra[i][j] = fmaf(mv[i][k], xv[k][j], intra[i][j]);
+        }
+        #pragma unroll
+        for (int i = 0; i < 4; i++)
+        {
+            if (t0 + i >= lc) break;
+            const float e = expf(s_cum[t0 + i]);
+            const f32x4 uv = *(const f32x4*)(a.u + (row0 + t0 + i) * a.ldu + h * P + p0);
+            f32x4 y;
+            #pragma unroll
+            for (int j = 0; j < 4; j++) y[j] = fmaf(e, inter[i][j], intra[i][j]) + Dh * uv[j];
+            *(f32x4*)(a.y + (row0 + t0 + i) * a.ldy + h * P + p0) = y;
+        }
+    }
+}
+
 // ---- gate + group-wise RMS norm -------------------------------------------------------------------------------------------------
 
 // grid (rows, norm groups): out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part]
@@ -284,6 +514,53 @@ extern "C" int exl2_ssm_scan(const float* u, int ldu, const float* B, const floa
     else if (npt <= 16) LAUNCH(scan_kernel<16>, grid, block, smem, stream, a);
     else if (npt <= 32) LAUNCH(scan_kernel<32>, grid, block, smem, stream, a);
     else LAUNCH(scan_kernel<SCAN_MAX_NPT>, grid, block, smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+static size_t ssd_out_smem(int N, int P)
+{
+    const size_t bs = (size_t)SSD_L * (N + 4) > (size_t)N * P ? (size_t)SSD_L * (N + 4) : (size_t)N * P;
+    return sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (N + 4) + bs + (size_t)SSD_L * P + (size_t)SSD_L * (SSD_L + 4));
+}
+
+/* 1 if exl2_ssm_scan_chunked takes this shape (sizes in fours that fit the LDS), 0 otherwise */
+extern "C" int exl2_ssm_scan_chunked_supported(int n_state, int vdim)
+{
+    return n_state > 0 && vdim > 0 && n_state % 4 == 0 && vdim % 4 == 0 && ssd_out_smem(n_state, vdim) <= 160 * 1024 - 256;
+}
+
+extern "C" int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
+                                     const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
+                                     const int* span_row0, const int* span_rows, const int* span_chunk0, int spans, int max_span_rows,
+                                     int chunk, const int* row_seq, const int* row_pos, float* zbuf, float* dbuf,
+                                     int heads, int groups, int n_state, int vdim, void* stream)
+{
+    EXL2_REQUIRE(u && B && C && dt && dt_bias && A_log && D && y && state && span_row0 && span_rows && span_chunk0 && row_seq && row_pos
+                 && zbuf && dbuf, "ssm_scan_chunked: null operand");
+    EXL2_REQUIRE(chunk == SSD_L, "ssm_scan_chunked: chunks of %d rows (the span table was made for %d)", SSD_L, chunk);
+    EXL2_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0, "ssm_scan_chunked: %d heads in %d groups", heads, groups);
+    EXL2_REQUIRE(exl2_ssm_scan_chunked_supported(n_state, vdim), "ssm_scan_chunked: state %d x %d outside the chunked form", n_state, vdim);
+    EXL2_REQUIRE(ldu % 4 == 0 && ldy % 4 == 0 && ((uintptr_t)u % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)zbuf % 16) == 0,
+                 "ssm_scan_chunked: rows of u / y must be 16-byte aligned");
+    if (spans <= 0 || max_span_rows <= 0) return EXL2_OK;
+    SsdArgs g;
+    ScanArgs& a = g.s;
+    a.u = u; a.ldu = ldu; a.B = B; a.C = C; a.ldbc = ldbc; a.dt = dt; a.lddt = lddt; a.dt_bias = dt_bias; a.A_log = A_log; a.D = D;
+    a.y = y; a.ldy = ldy; a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.groups = groups; a.N = n_state; a.P = vdim; a.KS = 0;
+    g.zbuf = zbuf; g.dbuf = dbuf; g.span_chunk0 = span_chunk0;
+    const size_t smem1 = sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (n_state + vdim)), smem3 = ssd_out_smem(n_state, vdim);
+    static bool attr_done[EXL2_MAX_DEVICES];
+    if (exl2_first_on_device(attr_done))
+    {
+        (void)hipFuncSetAttribute((const void*)ssd_chunk_state_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)ssd_chunk_out_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    }
+    const int chunks = (max_span_rows + SSD_L - 1) / SSD_L;
+    LAUNCH(ssd_chunk_state_kernel, dim3(chunks, heads, spans), dim3(256), smem1, stream, g);
+    LAUNCH(ssd_carry_kernel, dim3((n_state * vdim + 255) / 256, heads, spans), dim3(256), 0, stream, g);
+    LAUNCH(ssd_chunk_out_kernel, dim3(chunks, heads, spans), dim3(256), smem3, stream, g);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

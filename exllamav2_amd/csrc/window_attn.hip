@@ -17,6 +17,7 @@
 // Rotary layouts: halves (value i pairs with i + n / 2) or interleaved (2i with 2i + 1); angle p * freq[i], cos and sin times `amp`.
 #include "hw.h"
 #include "errors.h"
+#include <stdint.h>
 
 template <typename T> DEV float wa_ld(const T* p);
 template <> DEV float wa_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
@@ -132,11 +133,38 @@ struct PoolArgs
     int kw, vw;                              // values per token: G x dim, G x vdim
 };
 
-// grid (rows): a row whose position completes a block (pos % pool == pool - 1) writes that block's mean key and value row, read
-// back from the cache as it holds them; other rows leave at once.
-template <typename T>
+// 16 bytes of T as floats
+template <typename T> struct WaVec;
+template <> struct WaVec<u16>
+{
+    static constexpr int N = 8;
+    static DEV void load(const u16* p, float* f)
+    {
+        const u32x4 v = *(const u32x4*)p;
+        #pragma unroll
+        for (int i = 0; i < 4; i++) { f[2 * i] = as_f32(v[i] << 16); f[2 * i + 1] = as_f32(v[i] & 0xffff0000u); }
+    }
+};
+template <> struct WaVec<float>
+{
+    static constexpr int N = 4;
+    static DEV void load(const float* p, float* f)
+    {
+        const f32x4 v = *(const f32x4*)p;
+        #pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = v[i];
+    }
+};
+
+// grid (rows, pieces): a row whose position completes a block (pos % pool == pool - 1) writes that block's mean key and value row,
+// read back from the cache as it holds them; other rows leave at once.  VEC: a workgroup takes 64 16-byte pieces of the
+// [keys | values] row, wave w sums the block's tokens w, w + 4, .. and the four partial sums meet in LDS; otherwise one value per
+// thread over all tokens (sizes that are not whole 16-byte pieces).
+template <typename T, bool VEC>
 KERNEL void __launch_bounds__(256) pool_blocks_kernel(const PoolArgs a)
 {
+    constexpr int VN = WaVec<T>::N;
+    SHARED float part[4][64][VN];
     const int r = bid_x(), t = tid();
     const int pos = a.row_pos[r];
     if (pos % a.pool != a.pool - 1) return;
@@ -144,6 +172,36 @@ KERNEL void __launch_bounds__(256) pool_blocks_kernel(const PoolArgs a)
     const int p0 = pos - (a.pool - 1);
     const long long dst = (long long)bt[p0 / a.page] * a.per_page + (p0 % a.page) / a.pool;
     const float inv = 1.0f / (float)a.pool;
+    if (VEC)
+    {
+        const int w = wave_id(), lane = lane_id();
+        const int piece = bid_y() * 64 + lane, e0 = piece * VN;
+        const bool live = e0 < a.kw + a.vw;
+        const bool is_k = e0 < a.kw;
+        const int e = is_k ? e0 : e0 - a.kw, wd = is_k ? a.kw : a.vw;
+        const T* c = (const T*)(is_k ? a.k_cache : a.v_cache);
+        float acc[VN];
+        #pragma unroll
+        for (int i = 0; i < VN; i++) acc[i] = 0.0f;
+        if (live)
+            for (int j = p0 + w; j <= pos; j += 4)
+            {
+                float f[VN];
+                WaVec<T>::load(c + ((long long)bt[j / a.page] * a.page + j % a.page) * wd + e, f);
+                #pragma unroll
+                for (int i = 0; i < VN; i++) acc[i] += f[i];
+            }
+        #pragma unroll
+        for (int i = 0; i < VN; i++) part[w][lane][i] = acc[i];
+        block_sync();
+        if (w == 0 && live)
+        {
+            T* d = (T*)(is_k ? a.k_pool : a.v_pool) + dst * wd + e;
+            #pragma unroll
+            for (int i = 0; i < VN; i++) wa_st<T>(d + i, (part[0][lane][i] + part[1][lane][i] + part[2][lane][i] + part[3][lane][i]) * inv);
+        }
+        return;
+    }
     for (int i = t; i < a.kw + a.vw; i += 256)
     {
         const bool is_k = i < a.kw;
@@ -287,6 +345,507 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
     }
 }
 
+// ---- bfloat16 on the matrix cores ---------------------------------------------------------------------------------------------------
+// Workgroup = one tile of <= 64 consecutive positions of one sequence x one head; wave w owns the 16 query rows 16 w .. 16 w + 15.
+// The tile's key list is [pooled blocks 0 .. NB) | tokens j_lo .. last position], NB and j_lo taken for the tile as a whole and
+// masked per query row; it goes by in steps of 64 entries whose key and value rows are staged row-major in LDS (each entry's row is
+// looked up through the block table -- pooled rows in the pooled tensors -- one step ahead of its loads, two steps ahead of its use).
+// Scores are computed transposed, S^T = K Q^T (A = key rows from LDS, B = the wave's query rows held in registers), so that the
+// accumulator layout of S^T (lane (q, g) holds keys 4g .. 4g + 3 of a 16-key block for query q) is the B-operand layout of
+// O^T += V^T P^T with the 32 keys of a product taken in the order {4g .. 4g + 3 of block 0, of block 1}: probabilities stay in
+// registers, and V^T's A operand comes from the row-major value tile by transposing LDS reads.  Softmax statistics per query =
+// per accumulator column (running maximum starts at the sink, the sum at 1), fp32; P rounded to bfloat16 for the product.
+// The epilogue turns the head's output back by the row's position, applies the gate and stores bfloat16.
+
+struct WinMfmaArgs
+{
+    WinAttnArgs w;
+    const int* tile_row0; const int* tile_rows;
+};
+
+#define WM_BK 64
+#define WM_NEG_BIG (-1.0e30f)
+
+DEV u32 wm_pack2(float lo, float hi) { return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16); }
+
+template <int DIM, int VDIM>
+KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs m)
+{
+    DYN_SMEM(smem);
+    const WinAttnArgs& a = m.w;
+    constexpr int KSTR = DIM + 8, VSTR = VDIM + 16;              // row strides (values): conflict-free 16-byte and transposing reads
+    constexpr int KK = DIM / 32, DB = VDIM / 16, NBLK = WM_BK / 16;
+    constexpr int KP = WM_BK * DIM / 8, VP = WM_BK * VDIM / 8;   // 16-byte pieces of a key / value tile
+    constexpr int KPT = (KP + 255) / 256, VPT = (VP + 255) / 256;
+    u16* k_lds = (u16*)smem;
+    u16* v_lds = k_lds + WM_BK * KSTR;
+
+    const int t = tid(), lane = lane_id(), wv = wave_id();
+    const int qi = lane & 15, g = lane >> 4;
+    const int tile_i = bid_x(), h = bid_y();
+    const int kh = h / (a.H / a.G);
+    const int r0 = m.tile_row0[tile_i], n_rows = m.tile_rows[tile_i];
+    const int p0 = a.row_pos[r0], p_last = p0 + n_rows - 1;
+    const int* bt = a.block_table + (long long)a.row_seq[r0] * a.bt_stride;
+    const int NB = wa_blocks_seen(p_last, a.window, a.pool);
+    const int j_lo = max(0, p0 - a.window + 1);
+    const int total = NB + (p_last - j_lo + 1);
+    const int n_tiles = (total + WM_BK - 1) / WM_BK;
+    const u16* kc = (const u16*)a.k_cache; const u16* vc = (const u16*)a.v_cache;
+    const u16* kp = (const u16*)a.k_pool; const u16* vp = (const u16*)a.v_pool;
+
+    // entry e of the key list -> its row in the cache (>= 0) or in the pooled tensors (-1 - row)
+    auto entry_row = [&](int e) -> long long {
+        e = min(e, total - 1);
+        if (e < NB)
+        {
+            const int b0 = e * a.pool;
+            return -1 - ((long long)bt[b0 / a.page] * a.per_page + (b0 % a.page) / a.pool);
+        }
+        const int j = j_lo + (e - NB);
+        return (long long)bt[j / a.page] * a.page + j % a.page;
+    };
+
+    // this wave's 16 query rows as B operands: lane (qi, g) holds Q[row qi][32 kk + 8 g .. + 8]
+    const int my_row = wv * 16 + qi;
+    const int qrow = r0 + min(my_row, n_rows - 1);
+    const int qpos = p0 + min(my_row, n_rows - 1);
+    const bool wave_live = wv * 16 < n_rows;
+    u32x4 qb[KK];
+    {
+        const u16* qp = (const u16*)a.q + ((long long)qrow * a.H + h) * DIM + 8 * g;
+        #pragma unroll
+        for (int kk = 0; kk < KK; kk++) qb[kk] = *(const u32x4*)(qp + 32 * kk);
+    }
+    const int my_nb = wa_blocks_seen(qpos, a.window, a.pool);
+    const int my_lo = qpos - a.window + 1;                      // first token this query sees (may be negative)
+    // what the wave as a whole can see: blocks below wave_nb, tokens wave_lo .. wave_hi
+    const int wp0 = p0 + min(wv * 16, n_rows - 1), wp1 = p0 + min(wv * 16 + 15, n_rows - 1);
+    const int wave_nb = wa_blocks_seen(wp1, a.window, a.pool), wave_lo = wp0 - a.window + 1, wave_hi = wp1;
+
+    f32x4 ot[DB];
+    #pragma unroll
+    for (int d = 0; d < DB; d++) ot[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = a.sink ? a.sink[h] : WM_NEG_BIG, l_run = a.sink ? 1.0f : 0.0f;
+
+    long long krow[KPT], vrow[VPT];                             // rows of the NEXT step's pieces
+    u32x4 kreg[KPT], vreg[VPT];
+    auto lookup = [&](int step) {
+        const int k0 = step * WM_BK;
+        #pragma unroll
+        for (int i = 0; i < KPT; i++) krow[i] = entry_row(k0 + (t + i * 256) / (DIM / 8));
+        #pragma unroll
+        for (int i = 0; i < VPT; i++) vrow[i] = entry_row(k0 + (t + i * 256) / (VDIM / 8));
+    };
+    auto fetch = [&]() {
+        #pragma unroll
+        for (int i = 0; i < KPT; i++)
+        {
+            const int c = t + i * 256;
+            if (KP % 256 != 0 && c >= KP) break;
+            const long long row = krow[i];
+            const u16* src = row >= 0 ? kc + (row * a.G + kh) * DIM : kp + ((-1 - row) * a.G + kh) * DIM;
+            kreg[i] = *(const u32x4*)(src + (c % (DIM / 8)) * 8);
+        }
+        #pragma unroll
+        for (int i = 0; i < VPT; i++)
+        {
+            const int c = t + i * 256;
+            if (VP % 256 != 0 && c >= VP) break;
+            const long long row = vrow[i];
+            const u16* src = row >= 0 ? vc + (row * a.G + kh) * VDIM : vp + ((-1 - row) * a.G + kh) * VDIM;
+            vreg[i] = *(const u32x4*)(src + (c % (VDIM / 8)) * 8);
+        }
+    };
+    auto stage = [&]() {
+        #pragma unroll
+        for (int i = 0; i < KPT; i++)
+        {
+            const int c = t + i * 256;
+            if (KP % 256 != 0 && c >= KP) break;
+            *(u32x4*)(k_lds + (c / (DIM / 8)) * KSTR + (c % (DIM / 8)) * 8) = kreg[i];
+        }
+        #pragma unroll
+        for (int i = 0; i < VPT; i++)
+        {
+            const int c = t + i * 256;
+            if (VP % 256 != 0 && c >= VP) break;
+            *(u32x4*)(v_lds + (c / (VDIM / 8)) * VSTR + (c % (VDIM / 8)) * 8) = vreg[i];
+        }
+    };
+
+    lookup(0);
+    fetch();
+    if (n_tiles > 1) lookup(1);
+    for (int step = 0; step < n_tiles; step++)
+    {
+        block_sync();                                            // everybody is done with the previous step's tiles
+        stage();
+        block_sync();
+        if (step + 1 < n_tiles)
+        {
+            fetch();                                             // in flight during the products below
+            if (step + 2 < n_tiles) lookup(step + 2);
+        }
+        const int k0 = step * WM_BK;
+        // nothing in this step for the wave's rows?
+        {
+            const int e_hi = min(k0 + WM_BK, total) - 1;
+            bool any = false;
+            if (k0 < NB) any = k0 < wave_nb;
+            if (e_hi >= NB)
+            {
+                const int ja = j_lo + max(k0 - NB, 0), jb = j_lo + (e_hi - NB);
+                any = any || (ja <= wave_hi && jb >= wave_lo);
+            }
+            if (!wave_live || !any) continue;
+        }
+        f32x4 st[NBLK];
+        #pragma unroll
+        for (int blk = 0; blk < NBLK; blk++)
+        {
+            st[blk] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            const u16* kf = k_lds + (16 * blk + qi) * KSTR + 8 * g;
+            #pragma unroll
+            for (int kk = 0; kk < KK; kk++) st[blk] = mfma_16x16x32_bf16(*(const u32x4*)(kf + 32 * kk), qb[kk], st[blk]);
+        }
+        float sc[4 * NBLK];
+        float m_loc = WM_NEG_BIG;
+        #pragma unroll
+        for (int blk = 0; blk < NBLK; blk++)
+            #pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                const int e = k0 + 16 * blk + 4 * g + r;
+                const int j = j_lo + (e - NB);
+                const bool valid = e < total && (e < NB ? e < my_nb : (j <= qpos && j >= my_lo));
+                const float v = valid ? st[blk][r] : WM_NEG_BIG;
+                sc[blk * 4 + r] = v;
+                m_loc = fmaxf(m_loc, v);
+            }
+        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 16));
+        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 32));
+        const float m_new = fmaxf(m_run, m_loc);
+        const float alpha = expf(m_run - m_new);
+        float p_sum = 0.0f;
+        u32x4 pb[NBLK / 2];
+        #pragma unroll
+        for (int e2 = 0; e2 < 2 * NBLK; e2++)
+        {
+            const float pa = sc[2 * e2] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2] - m_new) : 0.0f;
+            const float pc = sc[2 * e2 + 1] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2 + 1] - m_new) : 0.0f;
+            p_sum += pa + pc;
+            pb[e2 / 4][e2 % 4] = wm_pack2(pa, pc);
+        }
+        p_sum += shfl_xor_f32(p_sum, 16);
+        p_sum += shfl_xor_f32(p_sum, 32);
+        l_run = l_run * alpha + p_sum;
+        m_run = m_new;
+        // O^T = alpha O^T + V^T P^T: this lane points at value row 4 g + qi / 4, features 16 d + 4 (qi % 4) .. + 3
+        const u16* vbase = v_lds + (4 * g + (qi >> 2)) * VSTR + 4 * (qi & 3);
+        #pragma unroll
+        for (int d = 0; d < DB; d++)
+        {
+            ot[d][0] *= alpha; ot[d][1] *= alpha; ot[d][2] *= alpha; ot[d][3] *= alpha;
+            #pragma unroll
+            for (int m2 = 0; m2 < NBLK / 2; m2++)
+            {
+                const f16x4 lo = lds_read_tr16_b64((const f16*)(vbase + (32 * m2) * VSTR + 16 * d));
+                const f16x4 hi = lds_read_tr16_b64((const f16*)(vbase + (32 * m2 + 16) * VSTR + 16 * d));
+                const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                ot[d] = mfma_16x16x32_bf16((u32x4){l2[0], l2[1], h2[0], h2[1]}, pb[m2], ot[d]);
+            }
+        }
+    }
+
+    // O^T[feature 16 d + 4 g + r][query qi] / l, turned back by the row's position, gated -> out[row][head][feature]
+    if (my_row >= n_rows) return;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    #pragma unroll
+    for (int d = 0; d < DB; d++) { ot[d][0] *= inv; ot[d][1] *= inv; ot[d][2] *= inv; ot[d][3] *= inv; }
+    if (a.v_rot)
+    {
+        const float fpos = (float)qpos;
+        if (a.interleaved)
+        {
+            #pragma unroll
+            for (int d = 0; d < DB; d++)
+                #pragma unroll
+                for (int r = 0; r < 4; r += 2)
+                {
+                    const float ang = fpos * a.vfreq[(16 * d + 4 * g + r) / 2];
+                    const float c = cosf(ang), sn = sinf(ang);
+                    const float u = ot[d][r], v = ot[d][r + 1];
+                    ot[d][r] = u * c + v * sn; ot[d][r + 1] = v * c - u * sn;
+                }
+        }
+        else
+        {
+            #pragma unroll
+            for (int d = 0; d < DB / 2; d++)
+                #pragma unroll
+                for (int r = 0; r < 4; r++)
+                {
+                    const float ang = fpos * a.vfreq[16 * d + 4 * g + r];
+                    const float c = cosf(ang), sn = sinf(ang);
+                    const float u = ot[d][r], v = ot[d + DB / 2][r];
+                    ot[d][r] = u * c + v * sn; ot[d + DB / 2][r] = v * c - u * sn;
+                }
+        }
+    }
+    u16* op = (u16*)a.out + ((long long)qrow * a.H + h) * VDIM + 4 * g;
+    const float* gt = a.gate ? a.gate + (long long)qrow * a.ldg + h * VDIM + 4 * g : nullptr;
+    #pragma unroll
+    for (int d = 0; d < DB; d++)
+    {
+        f32x4 y = ot[d];
+        if (gt)
+        {
+            const f32x4 gv = *(const f32x4*)(gt + 16 * d);
+            #pragma unroll
+            for (int r = 0; r < 4; r++) y[r] *= 1.0f / (1.0f + expf(-gv[r]));
+        }
+        *(u32x2*)(op + 16 * d) = (u32x2){wm_pack2(y[0], y[1]), wm_pack2(y[2], y[3])};
+    }
+}
+
+template <int DIM, int VDIM>
+static void wm_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
+{
+    static bool attr_done[EXL2_MAX_DEVICES];
+    const size_t lds = ((size_t)WM_BK * (DIM + 8) + (size_t)WM_BK * (VDIM + 16)) * 2;
+    if (exl2_first_on_device(attr_done))
+        (void)hipFuncSetAttribute((const void*)window_attn_mfma_kernel<DIM, VDIM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    LAUNCH((window_attn_mfma_kernel<DIM, VDIM>), dim3(tiles, m.w.H), dim3(256), lds, s, m);
+}
+
+// Decoded tokens: workgroup = one row x one key / value head.  The 16 query columns of the products are the query heads that
+// share the key head (at most 16 per workgroup; blockIdx.z walks further sixteens), all at the row's position, so the key list
+// [pooled blocks | window tokens] needs no mask beyond its length.  It goes by in steps of 128 entries staged by all four waves;
+// wave w takes entries 32 w .. 32 w + 31 of every step with its own running (maximum, sum, O^T) -- the sink counts in wave 0 --
+// and the four partial results meet in LDS at the end.  One pass over the keys serves all heads of the group.
+
+#define WD_BK 128
+
+template <int DIM, int VDIM>
+KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m)
+{
+    DYN_SMEM(smem);
+    const WinAttnArgs& a = m.w;
+    constexpr int KSTR = DIM + 8, VSTR = VDIM + 16;
+    constexpr int KK = DIM / 32, DB = VDIM / 16;
+    constexpr int KP = WD_BK * DIM / 8, VP = WD_BK * VDIM / 8;
+    constexpr int KPT = (KP + 255) / 256, VPT = (VP + 255) / 256;
+    u16* k_lds = (u16*)smem;
+    u16* v_lds = k_lds + WD_BK * KSTR;
+
+    const int t = tid(), lane = lane_id(), wv = wave_id();
+    const int qi = lane & 15, g = lane >> 4;
+    const int kh = bid_y();
+    const int hpg = a.H / a.G, h0 = bid_z() * 16, nh = min(16, hpg - h0);      // this workgroup's heads: kh * hpg + h0 .. + nh
+    const int r = m.tile_row0[bid_x()];
+    const int pos = a.row_pos[r];
+    const int* bt = a.block_table + (long long)a.row_seq[r] * a.bt_stride;
+    const int NB = wa_blocks_seen(pos, a.window, a.pool);
+    const int j_lo = max(0, pos - a.window + 1);
+    const int total = NB + (pos - j_lo + 1);
+    const int n_steps = (total + WD_BK - 1) / WD_BK;
+    const u16* kc = (const u16*)a.k_cache; const u16* vc = (const u16*)a.v_cache;
+    const u16* kp = (const u16*)a.k_pool; const u16* vp = (const u16*)a.v_pool;
+    auto entry_row = [&](int e) -> long long {
+        e = min(e, total - 1);
+        if (e < NB)
+        {
+            const int b0 = e * a.pool;
+            return -1 - ((long long)bt[b0 / a.page] * a.per_page + (b0 % a.page) / a.pool);
+        }
+        const int j = j_lo + (e - NB);
+        return (long long)bt[j / a.page] * a.page + j % a.page;
+    };
+    const int head = kh * hpg + h0 + min(qi, nh - 1);
+    u32x4 qb[KK];
+    {
+        const u16* qp = (const u16*)a.q + ((long long)r * a.H + head) * DIM + 8 * g;
+        #pragma unroll
+        for (int kk = 0; kk < KK; kk++) qb[kk] = *(const u32x4*)(qp + 32 * kk);
+    }
+    f32x4 ot[DB];
+    #pragma unroll
+    for (int d = 0; d < DB; d++) ot[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = (a.sink && wv == 0) ? a.sink[head] : WM_NEG_BIG, l_run = (a.sink && wv == 0) ? 1.0f : 0.0f;
+
+    long long krow[KPT], vrow[VPT];
+    u32x4 kreg[KPT], vreg[VPT];
+    auto lookup = [&](int step) {
+        const int k0 = step * WD_BK;
+        #pragma unroll
+        for (int i = 0; i < KPT; i++) krow[i] = entry_row(k0 + (t + i * 256) / (DIM / 8));
+        #pragma unroll
+        for (int i = 0; i < VPT; i++) vrow[i] = entry_row(k0 + (t + i * 256) / (VDIM / 8));
+    };
+    auto fetch = [&]() {
+        #pragma unroll
+        for (int i = 0; i < KPT; i++)
+        {
+            const int c = t + i * 256;
+            const long long row = krow[i];
+            const u16* src = row >= 0 ? kc + (row * a.G + kh) * DIM : kp + ((-1 - row) * a.G + kh) * DIM;
+            kreg[i] = *(const u32x4*)(src + (c % (DIM / 8)) * 8);
+        }
+        #pragma unroll
+        for (int i = 0; i < VPT; i++)
+        {
+            const int c = t + i * 256;
+            const long long row = vrow[i];
+            const u16* src = row >= 0 ? vc + (row * a.G + kh) * VDIM : vp + ((-1 - row) * a.G + kh) * VDIM;
+            vreg[i] = *(const u32x4*)(src + (c % (VDIM / 8)) * 8);
+        }
+    };
+    auto stage = [&]() {
+        #pragma unroll
+        for (int i = 0; i < KPT; i++)
+        {
+            const int c = t + i * 256;
+            *(u32x4*)(k_lds + (c / (DIM / 8)) * KSTR + (c % (DIM / 8)) * 8) = kreg[i];
+        }
+        #pragma unroll
+        for (int i = 0; i < VPT; i++)
+        {
+            const int c = t + i * 256;
+            *(u32x4*)(v_lds + (c / (VDIM / 8)) * VSTR + (c % (VDIM / 8)) * 8) = vreg[i];
+        }
+    };
+    static_assert(KP % 256 == 0 && VP % 256 == 0, "a step is a whole number of 16-byte pieces per thread");
+
+    lookup(0);
+    fetch();
+    if (n_steps > 1) lookup(1);
+    for (int step = 0; step < n_steps; step++)
+    {
+        block_sync();
+        stage();
+        block_sync();
+        if (step + 1 < n_steps)
+        {
+            fetch();
+            if (step + 2 < n_steps) lookup(step + 2);
+        }
+        const int k0 = step * WD_BK + 32 * wv;                  // this wave's 32 entries
+        if (k0 >= total) continue;
+        f32x4 st[2];
+        #pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+        {
+            st[blk] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            const u16* kf = k_lds + (32 * wv + 16 * blk + qi) * KSTR + 8 * g;
+            #pragma unroll
+            for (int kk = 0; kk < KK; kk++) st[blk] = mfma_16x16x32_bf16(*(const u32x4*)(kf + 32 * kk), qb[kk], st[blk]);
+        }
+        float sc[8];
+        float m_loc = WM_NEG_BIG;
+        #pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+            #pragma unroll
+            for (int rr = 0; rr < 4; rr++)
+            {
+                const float v = k0 + 16 * blk + 4 * g + rr < total ? st[blk][rr] : WM_NEG_BIG;
+                sc[blk * 4 + rr] = v;
+                m_loc = fmaxf(m_loc, v);
+            }
+        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 16));
+        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 32));
+        const float m_new = fmaxf(m_run, m_loc);
+        const float alpha = expf(m_run - m_new);
+        float p_sum = 0.0f;
+        u32x4 pb;
+        #pragma unroll
+        for (int e2 = 0; e2 < 4; e2++)
+        {
+            const float pa = sc[2 * e2] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2] - m_new) : 0.0f;
+            const float pc = sc[2 * e2 + 1] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2 + 1] - m_new) : 0.0f;
+            p_sum += pa + pc;
+            pb[e2] = wm_pack2(pa, pc);
+        }
+        p_sum += shfl_xor_f32(p_sum, 16);
+        p_sum += shfl_xor_f32(p_sum, 32);
+        l_run = l_run * alpha + p_sum;
+        m_run = m_new;
+        const u16* vbase = v_lds + (32 * wv + 4 * g + (qi >> 2)) * VSTR + 4 * (qi & 3);
+        #pragma unroll
+        for (int d = 0; d < DB; d++)
+        {
+            ot[d][0] *= alpha; ot[d][1] *= alpha; ot[d][2] *= alpha; ot[d][3] *= alpha;
+            const f16x4 lo = lds_read_tr16_b64((const f16*)(vbase + 16 * d));
+            const f16x4 hi = lds_read_tr16_b64((const f16*)(vbase + 16 * VSTR + 16 * d));
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            ot[d] = mfma_16x16x32_bf16((u32x4){l2[0], l2[1], h2[0], h2[1]}, pb, ot[d]);
+        }
+    }
+
+    // the four waves' partial results -> LDS (over the tiles): [wave][16 queries] (m, l), [wave][VDIM][16] O^T
+    block_sync();
+    float* s_ml = (float*)smem;                                  // [4][16][2]
+    float* s_o = s_ml + 4 * 16 * 2;                              // [4][VDIM][16]
+    if (g == 0) { s_ml[(wv * 16 + qi) * 2] = m_run; s_ml[(wv * 16 + qi) * 2 + 1] = l_run; }
+    #pragma unroll
+    for (int d = 0; d < DB; d++)
+        #pragma unroll
+        for (int rr = 0; rr < 4; rr++) s_o[(wv * VDIM + 16 * d + 4 * g + rr) * 16 + qi] = ot[d][rr];
+    block_sync();
+    // thread = (query column, pair of values): merge, turn back, gate, store
+    const float fpos = (float)pos;
+    for (int i = t; i < 16 * (VDIM / 2); i += 256)
+    {
+        const int q = i % 16, pr = i / 16;
+        if (q >= nh) continue;
+        int ia, ib;
+        wa_pair(pr, VDIM, a.interleaved, ia, ib);
+        float mx = WM_NEG_BIG;
+        #pragma unroll
+        for (int w = 0; w < 4; w++) mx = fmaxf(mx, s_ml[(w * 16 + q) * 2]);
+        float l = 0.0f, u = 0.0f, v = 0.0f;
+        #pragma unroll
+        for (int w = 0; w < 4; w++)
+        {
+            const float mw = s_ml[(w * 16 + q) * 2];
+            const float sc2 = mw > 0.5f * WM_NEG_BIG ? expf(mw - mx) : 0.0f;
+            l = fmaf(s_ml[(w * 16 + q) * 2 + 1], sc2, l);
+            u = fmaf(s_o[(w * VDIM + ia) * 16 + q], sc2, u);
+            v = fmaf(s_o[(w * VDIM + ib) * 16 + q], sc2, v);
+        }
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        u *= inv; v *= inv;
+        if (a.v_rot)
+        {
+            const float ang = fpos * a.vfreq[pr];
+            const float c = cosf(ang), sn = sinf(ang);
+            const float u2 = u * c + v * sn, v2 = v * c - u * sn;
+            u = u2; v = v2;
+        }
+        const int hd = kh * hpg + h0 + q;
+        if (a.gate)
+        {
+            const float* gt = a.gate + (long long)r * a.ldg + hd * VDIM;
+            u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib]));
+        }
+        u16* op = (u16*)a.out + ((long long)r * a.H + hd) * VDIM;
+        op[ia] = f32_to_bf16(u); op[ib] = f32_to_bf16(v);
+    }
+}
+
+template <int DIM, int VDIM>
+static void wd_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
+{
+    static bool attr_done[EXL2_MAX_DEVICES];
+    size_t lds = ((size_t)WD_BK * (DIM + 8) + (size_t)WD_BK * (VDIM + 16)) * 2;
+    const size_t merge = sizeof(float) * (4 * 16 * 2 + (size_t)4 * VDIM * 16);
+    if (merge > lds) lds = merge;
+    if (exl2_first_on_device(attr_done))
+        (void)hipFuncSetAttribute((const void*)window_attn_decode_kernel<DIM, VDIM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    const int hpg = m.w.H / m.w.G;
+    LAUNCH((window_attn_decode_kernel<DIM, VDIM>), dim3(tiles, m.w.G, (hpg + 15) / 16), dim3(256), lds, s, m);
+}
+
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
 
 extern "C" int exl2_kv_rot_append(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
@@ -315,8 +874,11 @@ extern "C" int exl2_kv_rot_append(const float* f, int ld, int q_off, int k_off, 
         p.k_cache = k_cache; p.v_cache = v_cache; p.k_pool = k_pool; p.v_pool = v_pool; p.row_seq = row_seq; p.row_pos = row_pos;
         p.block_table = block_table; p.bt_stride = bt_stride; p.page = page; p.pool = pool; p.per_page = (page + pool - 1) / pool;
         p.kw = kv_heads * dim; p.vw = kv_heads * vdim;
-        if (dtype == 0) LAUNCH(pool_blocks_kernel<u16>, dim3(rows), dim3(256), 0, stream, p);
-        else LAUNCH(pool_blocks_kernel<float>, dim3(rows), dim3(256), 0, stream, p);
+        const int vn = dtype == 0 ? 8 : 4;
+        const bool vec = p.kw % vn == 0 && p.vw % vn == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0;
+        const dim3 grid(rows, vec ? ((p.kw + p.vw) / vn + 63) / 64 : 1);
+        if (dtype == 0) { if (vec) LAUNCH((pool_blocks_kernel<u16, true>), grid, dim3(256), 0, stream, p); else LAUNCH((pool_blocks_kernel<u16, false>), grid, dim3(256), 0, stream, p); }
+        else { if (vec) LAUNCH((pool_blocks_kernel<float, true>), grid, dim3(256), 0, stream, p); else LAUNCH((pool_blocks_kernel<float, false>), grid, dim3(256), 0, stream, p); }
     }
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
@@ -342,6 +904,66 @@ extern "C" int exl2_window_attn(const void* q, const void* k_cache, const void* 
     const size_t smem = (size_t)(dim + vdim) * 4;
     if (dtype == 0) LAUNCH(window_attn_kernel<u16>, dim3(rows, heads), dim3(256), smem, stream, a);
     else LAUNCH(window_attn_kernel<float>, dim3(rows, heads), dim3(256), smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+/* 1 if exl2_window_attn_tiles takes these head sizes */
+extern "C" int exl2_window_attn_tiles_supported(int dim, int vdim)
+{
+    return (dim == vdim && (dim == 32 || dim == 64 || dim == 96 || dim == 128 || dim == 256)) || (dim == 192 && vdim == 128)
+           || (dim == 128 && vdim == 64) || (dim == 64 && vdim == 128);
+}
+
+/* exl2_window_attn on the matrix cores (bfloat16, head sizes of exl2_window_attn_tiles_supported; gate rows and offsets multiples
+   of 4 values).  The step's rows come as tiles.  tile_mode 64: tile i = rows tile_row0[i] .. + tile_rows[i], <= 64 consecutive
+   positions of ONE sequence (portions of prompts; one head per workgroup).  tile_mode 1: the single rows tile_row0[i] (decoded
+   tokens; the heads of a key / value head share one pass over the keys). */
+extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                      const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                                      const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                                      void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, int heads,
+                                      int kv_heads, int dim, int vdim, int window, void* stream)
+{
+    EXL2_REQUIRE(q && k_cache && v_cache && row_seq && row_pos && block_table && out && tile_row0, "window_attn_tiles: null operand");
+    EXL2_REQUIRE(tile_mode == 64 || tile_mode == 1, "window_attn_tiles: tile_mode is 64 or 1");
+    EXL2_REQUIRE(tile_mode == 1 || tile_rows, "window_attn_tiles: tile_rows missing");
+    EXL2_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "window_attn_tiles: bad head shape");
+    EXL2_REQUIRE(page > 0 && window > 0 && pool >= 0 && (pool == 0 || (k_pool && v_pool)), "window_attn_tiles: bad window / paging");
+    EXL2_REQUIRE(!v_rot || vfreq, "window_attn_tiles: rotated values need their frequencies");
+    EXL2_REQUIRE(!gate || (ldg % 4 == 0 && ((uintptr_t)gate % 16) == 0), "window_attn_tiles: gate rows must be 16-byte aligned");
+    if (!exl2_window_attn_tiles_supported(dim, vdim))
+        EXL2_FAIL(EXL2_E_UNSUPPORTED, "window_attn_tiles: head sizes %d / %d outside the matrix-core form", dim, vdim);
+    if (tiles <= 0) return EXL2_OK;
+    WinMfmaArgs m;
+    WinAttnArgs& a = m.w;
+    a.q = q; a.k_cache = k_cache; a.v_cache = v_cache; a.k_pool = k_pool; a.v_pool = v_pool; a.sink = sink; a.gate = gate; a.ldg = ldg;
+    a.vfreq = vfreq; a.v_rot = v_rot; a.interleaved = interleaved; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table;
+    a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
+    a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window;
+    m.tile_row0 = tile_row0; m.tile_rows = tile_rows;
+    hipStream_t s = (hipStream_t)stream;
+    if (tile_mode == 1)
+    {
+        if (dim == 32 && vdim == 32) wd_launch<32, 32>(m, tiles, s);
+        else if (dim == 64 && vdim == 64) wd_launch<64, 64>(m, tiles, s);
+        else if (dim == 96 && vdim == 96) wd_launch<96, 96>(m, tiles, s);
+        else if (dim == 128 && vdim == 128) wd_launch<128, 128>(m, tiles, s);
+        else if (dim == 256 && vdim == 256) wd_launch<256, 256>(m, tiles, s);
+        else if (dim == 192 && vdim == 128) wd_launch<192, 128>(m, tiles, s);
+        else if (dim == 128 && vdim == 64) wd_launch<128, 64>(m, tiles, s);
+        else wd_launch<64, 128>(m, tiles, s);
+        HIP_TRY(hipGetLastError());
+        return EXL2_OK;
+    }
+    if (dim == 32 && vdim == 32) wm_launch<32, 32>(m, tiles, s);
+    else if (dim == 64 && vdim == 64) wm_launch<64, 64>(m, tiles, s);
+    else if (dim == 96 && vdim == 96) wm_launch<96, 96>(m, tiles, s);
+    else if (dim == 128 && vdim == 128) wm_launch<128, 128>(m, tiles, s);
+    else if (dim == 256 && vdim == 256) wm_launch<256, 256>(m, tiles, s);
+    else if (dim == 192 && vdim == 128) wm_launch<192, 128>(m, tiles, s);
+    else if (dim == 128 && vdim == 64) wm_launch<128, 64>(m, tiles, s);
+    else wm_launch<64, 128>(m, tiles, s);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

@@ -12,7 +12,7 @@ import random
 import torch
 
 from .cache import PAGE_SIZE, PagePool
-from .layered import StepBatch
+from .layered import SPAN_CHUNK, StepBatch
 
 
 class Engine:
@@ -41,6 +41,7 @@ class Engine:
         back after the step.  Returns fp32 logits [n wanted, vocab] on the device, or None."""
         ids, seq, pos, want_rows = [], [], [], []
         t16_row0, t16_rows, t1_row0, t1_maxpos = [], [], [], 0
+        t64_row0, t64_rows = [], []
         spans = []
         seen = set()
         for rid, tokens, want in entries:
@@ -56,6 +57,9 @@ class Engine:
             start = self.pool.extend(slot, n)
             base = len(ids)
             spans.append((base, n, slot, start))
+            for i in range(0, n if n > 1 else 0, 64):
+                t64_row0.append(base + i)
+                t64_rows.append(min(64, n - i))
             if n == 1:
                 t1_row0.append(base)
                 t1_maxpos = max(t1_maxpos, start)
@@ -78,8 +82,16 @@ class Engine:
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
             batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows), spans=spans)
-            sp = torch.tensor([[s[0] for s in spans], [s[1] for s in spans]], dtype=torch.int32).to(dev)
+            chunk0, total = [], 0
+            for s in spans:                                       # recurrent mixers unroll long spans in chunks of SPAN_CHUNK rows
+                chunk0.append(total)
+                total += -(-s[1] // SPAN_CHUNK)
+            sp = torch.tensor([[s[0] for s in spans], [s[1] for s in spans], chunk0], dtype=torch.int32).to(dev)
             batch.spans_dev = (sp[0], sp[1], len(spans), max(s[1] for s in spans))
+            batch.span_chunks = (sp[2], SPAN_CHUNK, total)
+            if t64_row0:
+                t64 = torch.tensor([t64_row0, t64_rows], dtype=torch.int32).to(dev)
+                batch.tiles64 = (t64[0], t64[1], len(t64_row0))
             if t16_row0:
                 t16 = torch.tensor([t16_row0, t16_rows], dtype=torch.int32).to(dev)
                 batch.tiles16 = (t16[0], t16[1], len(t16_row0))

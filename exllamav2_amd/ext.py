@@ -922,6 +922,25 @@ class ExtC:
                                               self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(groups), int(n_state), int(vdim),
                                               self._stream(y)))
 
+    def ssm_scan_chunked_supported(self, n_state: int, vdim: int) -> bool:
+        return bool(self.lib.exl2_ssm_scan_chunked_supported(int(n_state), int(vdim)))
+
+    def ssm_scan_chunked(self, c, ldc: int, u_off: int, b_off: int, c_off: int, f, ldf: int, dt_off: int, dt_bias, a_log, d, y, state, spans,
+                         chunks, row_seq, row_pos, zbuf, dbuf, heads: int, groups: int, n_state: int, vdim: int) -> None:
+        """ssm_scan in chunks; chunks = (span_chunk0 int32 [n], chunk size, chunks in all): zbuf / dbuf hold one entry per chunk"""
+        row0, nrows, n, longest = spans
+        chunk0, chunk, total = chunks
+        if zbuf.numel() < total * heads * n_state * vdim or dbuf.numel() < total * heads:
+            raise RuntimeError("ssm_scan_chunked: scratch smaller than the step's chunks")
+        cp, fp = self._ptr(c, torch.float32, "c"), self._ptr(f, torch.float32, "f")
+        self.lib.check(self.lib.exl2_ssm_scan_chunked(
+            cp + u_off * 4, int(ldc), cp + b_off * 4, cp + c_off * 4, int(ldc), fp + dt_off * 4, int(ldf),
+            self._ptr(dt_bias, torch.float32, "dt_bias"), self._ptr(a_log, torch.float32, "A_log"), self._ptr(d, torch.float32, "D"),
+            self._ptr(y, torch.float32, "y"), y.shape[-1], self._ptr(state, torch.float32, "state"), self._ptr(row0, torch.int32, "span_row0"),
+            self._ptr(nrows, torch.int32, "span_rows"), self._ptr(chunk0, torch.int32, "span_chunk0"), int(n), int(longest), int(chunk),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(zbuf, torch.float32, "zbuf"),
+            self._ptr(dbuf, torch.float32, "dbuf"), int(heads), int(groups), int(n_state), int(vdim), self._stream(y)))
+
     def gated_group_norm(self, y, z, ldz: int, w, out, rows: int, dim: int, groups: int, eps: float) -> None:
         """out = rms_per_group(y * silu(z)) * w; y fp32 [rows, dim], z fp32 rows of leading dimension ldz (first dim columns)"""
         self.lib.check(self.lib.exl2_gated_group_norm(self._ptr(y, torch.float32, "y"), y.shape[-1], self._ptr(z, torch.float32, "z"), int(ldz),
@@ -955,6 +974,25 @@ class ExtC:
             int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
             self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, dt, "out"),
             self._dense_code(dt), int(rows), int(heads), int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
+
+    def window_attn_tiles_supported(self, dtype, dim: int, vdim: int) -> bool:
+        return dtype is torch.bfloat16 and bool(self.lib.exl2_window_attn_tiles_supported(int(dim), int(vdim)))
+
+    def window_attn_tiles(self, q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg: int, gate_off: int, vfreq, v_rot: bool,
+                          interleaved: bool, row_seq, row_pos, block_table, page: int, pool: int, out, tiles, tile_mode: int, heads: int,
+                          kv_heads: int, dim: int, vdim: int, window: int) -> None:
+        """tile_mode 64: tiles = (tile_row0 int32 [n], tile_rows int32 [n], n), runs of <= 64 consecutive positions of one sequence;
+        tile_mode 1: tiles = (rows int32 [n], None, n), single decoded rows"""
+        row0, nrows, n = tiles
+        bf = torch.bfloat16
+        gp = None if gate is None else self._ptr(gate, torch.float32, "gate") + gate_off * 4
+        self.lib.check(self.lib.exl2_window_attn_tiles(
+            self._ptr(q, bf, "q"), self._ptr(k_cache, bf, "k_cache"), self._ptr(v_cache, bf, "v_cache"), self._ptr(k_pool, bf, "k_pool"),
+            self._ptr(v_pool, bf, "v_pool"), self._ptr(sink, torch.float32, "sink"), gp, int(ldg), self._ptr(vfreq, torch.float32, "vfreq"),
+            int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+            self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, bf, "out"),
+            self._ptr(row0, torch.int32, "tile_row0"), self._ptr(nrows, torch.int32, "tile_rows"), int(n), int(tile_mode), int(heads),
+            int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
 
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))

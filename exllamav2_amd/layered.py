@@ -67,6 +67,9 @@ MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention,
 FEED_FORWARDS = {"dense": _dense_mlp, "moe": _moe_mlp}       # config `mlp.kind` -> builder(model, key, layer index, mlp spec)
 
 
+SPAN_CHUNK = 64                                           # rows per chunk of the chunked scan (csrc/ssm.hip: SSD_L)
+
+
 @dataclass
 class StepBatch:
     """Device-side description of one step: int32 tensors ids / row_seq / row_pos [rows], block_table [slots, pages],
@@ -82,9 +85,13 @@ class StepBatch:
     # (row0 int32 [n], rows int32 [n], n) and single decoded tokens (row0 int32 [n], n, largest position among them)
     tiles16: tuple | None = None
     tiles1: tuple | None = None
+    # the portions of prompts again in tiles of <= 64 consecutive positions (row0 int32 [n], rows int32 [n], n)
+    tiles64: tuple | None = None
     # the runs of consecutive rows that one sequence brings (recurrent mixers walk them in order): (first row int32 [n],
     # rows int32 [n], n, longest run)
     spans_dev: tuple | None = None
+    # the spans cut into chunks of SPAN_CHUNK rows: (number of chunks in front of each span int32 [n], SPAN_CHUNK, chunks in all)
+    span_chunks: tuple | None = None
     # host-side view of the same rows, one tuple per request in the step: (first row, rows, sequence slot, first position)
     spans: list | None = None
 

@@ -17,6 +17,8 @@ from .dense_linear import DenseLinear
 
 
 class StateSpaceMixer:
+    CHUNKED_FROM = 8                                          # longest span of a step from which the chunked scan is taken
+
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, vdim: int, state: int, groups: int, norm_groups: int, taps: int):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
         self.heads, self.vdim, self.state, self.groups, self.norm_groups, self.taps = heads, vdim, state, groups, norm_groups, taps
@@ -25,6 +27,7 @@ class StateSpaceMixer:
         if heads % groups or self.inner % norm_groups:
             raise ValueError(f"{key}: {heads} heads in {groups} groups, {self.inner} values in {norm_groups} norm groups")
         self.kv_from = None
+        self.chunked_ok = self.ext.ssm_scan_chunked_supported(state, vdim) and self.inner % 4 == 0 and self.channels % 4 == 0
 
     def load(self, get):
         """`get(name)` returns the device tensor `<layer>.mix.<name>` in the model's operand dtype"""
@@ -57,8 +60,18 @@ class StateSpaceMixer:
         ext.conv_silu_rows(f, self.n_front, inner, self.conv_w, self.conv_b, c, st["tail"], batch.spans_dev, batch.row_seq, batch.row_pos,
                            self.channels, self.taps)
         y = m.buf("ssm.y", (rows, inner), f32)
-        ext.ssm_scan(c, self.channels, 0, inner, inner + gn, f, self.n_front, 2 * inner + 2 * gn, self.dt_bias, self.a_log, self.d, y,
-                     st["S"], batch.spans_dev, batch.row_seq, batch.row_pos, self.heads, self.groups, self.state, self.vdim)
+        scan_args = (c, self.channels, 0, inner, inner + gn, f, self.n_front, 2 * inner + 2 * gn, self.dt_bias, self.a_log, self.d, y, st["S"],
+                     batch.spans_dev)
+        if batch.span_chunks is not None and batch.spans_dev[3] >= self.CHUNKED_FROM and self.chunked_ok:
+            # portions of prompts: the recurrence unrolled in chunks, every (chunk, head) independent work
+            total = batch.span_chunks[2]
+            zbuf = m.buf("ssm.z", (total, self.heads, self.state, self.vdim), f32)
+            dbuf = m.buf("ssm.d", (total, self.heads), f32)
+            ext.ssm_scan_chunked(*scan_args, batch.span_chunks, batch.row_seq, batch.row_pos, zbuf, dbuf, self.heads, self.groups,
+                                 self.state, self.vdim)
+        else:
+            # decoded tokens and short portions: one pass per (span, head) with the state in registers
+            ext.ssm_scan(*scan_args, batch.row_seq, batch.row_pos, self.heads, self.groups, self.state, self.vdim)
         g = m.buf("ssm.g", (rows, inner), m.dtype)
         ext.gated_group_norm(y, f, self.n_front, self.norm_w, g, rows, inner, self.norm_groups, m.norm_eps)
         return self.o.forward(g, rows, out=m.buf("mix.y", (rows, m.width), f32))

@@ -54,6 +54,7 @@ class WindowAttention:
         if heads % kv_heads or rot_dims > dim or rot_dims % 2 or (rotate_values and vdim % 2) or window <= 0 or pool < 0:
             raise ValueError(f"{key}: inconsistent attention sizes")
         self.kv_from = None
+        self.tiles_ok = self.ext.window_attn_tiles_supported(model.dtype, dim, vdim) and (self.heads * vdim) % 4 == 0
 
     def load(self, get):
         """`get(name)` returns the device tensor `<layer>.mix.<name>` in the model's operand dtype"""
@@ -96,7 +97,15 @@ class WindowAttention:
                           self.rot_dims, self.vfreq, self.rotate_values, self.interleaved, batch.row_seq, batch.row_pos, batch.block_table,
                           page, self.pool, rows, H, G, dim, vd)
         o = m.buf("attn.o", (rows, H * vd), m.dtype)
-        ext.window_attn(q, st.k, st.v, st.k_pool, st.v_pool, self.sink, f, ncat, self.off_g, self.vfreq, self.rotate_values,
-                        self.interleaved, batch.row_seq, batch.row_pos, batch.block_table, page, self.pool, o, rows, H, G, dim, vd,
-                        self.window)
+        common = (q, st.k, st.v, st.k_pool, st.v_pool, self.sink, f, ncat, self.off_g, self.vfreq, self.rotate_values, self.interleaved,
+                  batch.row_seq, batch.row_pos, batch.block_table, page, self.pool, o)
+        if self.tiles_ok and (batch.tiles64 is not None or batch.tiles1 is not None):
+            # matrix-core kernels: portions of prompts as tiles of <= 64 positions x one head per workgroup, decoded tokens as one row x
+            # one key / value head per workgroup (its query heads share the pass over the keys)
+            if batch.tiles64 is not None:
+                ext.window_attn_tiles(*common, batch.tiles64, 64, H, G, dim, vd, self.window)
+            if batch.tiles1 is not None:
+                ext.window_attn_tiles(*common, (batch.tiles1[0], None, batch.tiles1[1]), 1, H, G, dim, vd, self.window)
+        else:
+            ext.window_attn(*common, rows, H, G, dim, vd, self.window)
         return self.o.forward(o, rows, out=m.buf("mix.y", (rows, m.width), f32))

@@ -466,6 +466,16 @@ int exl2_ssm_scan(const float* u, int ldu, const float* B, const float* C, int l
                   const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
                   const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
                   int heads, int groups, int n_state, int vdim, void* stream);
+/* exl2_ssm_scan for portions of prompts: the recurrence unrolled in chunks of `chunk` (64) rows, every (chunk, head) independent
+   work around a short carry over each span's chunks.  span_chunk0[i] = number of chunks of the spans before i; zbuf fp32
+   [all chunks, heads, n_state, vdim] and dbuf fp32 [all chunks, heads] are scratch.  n_state and vdim multiples of 4 that fit the
+   LDS (exl2_ssm_scan_chunked_supported), rows of u / y 16-byte aligned. */
+int exl2_ssm_scan_chunked_supported(int n_state, int vdim);
+int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
+                          const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
+                          const int* span_row0, const int* span_rows, const int* span_chunk0, int spans, int max_span_rows,
+                          int chunk, const int* row_seq, const int* row_pos, float* zbuf, float* dbuf,
+                          int heads, int groups, int n_state, int vdim, void* stream);
 /* out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part] for each of `groups` equal parts of the dim values */
 int exl2_gated_group_norm(const float* y, int ldy, const float* z, int ldz, const void* w, void* out, int ldo, int out_f32,
                           int dtype, int rows, int dim, int groups, float eps, void* stream);
@@ -490,6 +500,17 @@ int exl2_window_attn(const void* q, const void* k_cache, const void* v_cache, co
                      const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
                      const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
                      void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, void* stream);
+
+/* exl2_window_attn on the matrix cores: bfloat16, head sizes for which exl2_window_attn_tiles_supported returns 1 (others:
+   EXL2_E_UNSUPPORTED), gate rows 16-byte aligned.  The step's rows come as tiles.  tile_mode 64: tile i = rows tile_row0[i] ..
+   + tile_rows[i], at most 64 consecutive positions of ONE sequence (portions of prompts).  tile_mode 1: the single rows
+   tile_row0[i] (decoded tokens: the query heads of a key / value head share one pass over the keys). */
+int exl2_window_attn_tiles_supported(int dim, int vdim);
+int exl2_window_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                           const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                           const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                           void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, int heads,
+                           int kv_heads, int dim, int vdim, int window, void* stream);
 
 #ifdef __cplusplus
 }
