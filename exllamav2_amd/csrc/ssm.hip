@@ -442,27 +442,56 @@ KERNEL void __launch_bounds__(256) ssd_chunk_out_kernel(const SsdArgs g)
 
 // ---- gate + group-wise RMS norm -------------------------------------------------------------------------------------------------
 
-// grid (rows, norm groups): out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part]
+// grid (rows, norm groups): out[r, part] = rms(y[r, part] * silu(z[r, part])) * w[part].  Parts of up to 256 * GN_EPT values are held in
+// registers between the two passes (all of a thread's loads leave together); longer parts are read twice.
+#define GN_EPT 16
+
 template <typename T>
 KERNEL void __launch_bounds__(256) gated_group_norm_kernel(const float* y, int ldy, const float* z, int ldz, const T* w, void* out, int ldo,
                                                             int out_f32, int part, float eps)
 {
     SHARED float red[4];
     const int r = bid_x(), o0 = bid_y() * part;
+    const float* yr = y + (long long)r * ldy + o0;
+    const float* zr = z + (long long)r * ldz + o0;
+    const bool held = part <= 256 * GN_EPT;
+    float v[GN_EPT];
     float ss = 0.0f;
-    for (int i = tid(); i < part; i += 256)
+    if (held)
     {
-        const float v = y[(long long)r * ldy + o0 + i] * ss_silu(z[(long long)r * ldz + o0 + i]);
-        ss = fmaf(v, v, ss);
+        float yv[GN_EPT], zv[GN_EPT];
+        #pragma unroll
+        for (int e = 0; e < GN_EPT; e++)
+        {
+            const int i = tid() + 256 * e;
+            yv[e] = i < part ? yr[i] : 0.0f;
+            zv[e] = i < part ? zr[i] : 0.0f;
+        }
+        #pragma unroll
+        for (int e = 0; e < GN_EPT; e++) { v[e] = yv[e] * ss_silu(zv[e]); ss = fmaf(v[e], v[e], ss); }
     }
+    else
+        for (int i = tid(); i < part; i += 256) { const float x = yr[i] * ss_silu(zr[i]); ss = fmaf(x, x, ss); }
     ss = wave_allreduce_add(ss);
     if (lane_id() == 0) red[wave_id()] = ss;
     block_sync();
     const float rinv = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)part + eps);
+    if (held)
+    {
+        #pragma unroll
+        for (int e = 0; e < GN_EPT; e++)
+        {
+            const int i = tid() + 256 * e;
+            if (i >= part) break;
+            const float o = v[e] * rinv * ss_ld<T>(w + o0 + i);
+            if (out_f32) ((float*)out)[(long long)r * ldo + o0 + i] = o; else ss_st<T>((T*)out + (long long)r * ldo + o0 + i, o);
+        }
+        return;
+    }
     for (int i = tid(); i < part; i += 256)
     {
-        const float v = y[(long long)r * ldy + o0 + i] * ss_silu(z[(long long)r * ldz + o0 + i]) * rinv * ss_ld<T>(w + o0 + i);
-        if (out_f32) ((float*)out)[(long long)r * ldo + o0 + i] = v; else ss_st<T>((T*)out + (long long)r * ldo + o0 + i, v);
+        const float o = yr[i] * ss_silu(zr[i]) * rinv * ss_ld<T>(w + o0 + i);
+        if (out_f32) ((float*)out)[(long long)r * ldo + o0 + i] = o; else ss_st<T>((T*)out + (long long)r * ldo + o0 + i, o);
     }
 }
 

@@ -225,7 +225,11 @@ struct WinAttnArgs
     const int* row_seq; const int* row_pos; const int* block_table; int bt_stride, page, pool, per_page;
     void* out;                               // [rows, H, vdim]
     int H, G, dim, vdim, window;
+    int page_shift, pool_shift;              // log2 of page / pool where they are powers of two, else -1 (tile kernels: no divisions)
 };
+
+DEV int wa_div(int x, int d, int shift) { return shift >= 0 ? x >> shift : x / d; }
+DEV int wa_mod(int x, int d, int shift) { return shift >= 0 ? x & (d - 1) : x % d; }
 
 #define WA_MAX_V_PER_THREAD 4
 
@@ -400,10 +404,11 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
         if (e < NB)
         {
             const int b0 = e * a.pool;
-            return -1 - ((long long)bt[b0 / a.page] * a.per_page + (b0 % a.page) / a.pool);
+            return -1 - ((long long)bt[wa_div(b0, a.page, a.page_shift)] * a.per_page
+                         + wa_div(wa_mod(b0, a.page, a.page_shift), a.pool, a.pool_shift));
         }
         const int j = j_lo + (e - NB);
-        return (long long)bt[j / a.page] * a.page + j % a.page;
+        return (long long)bt[wa_div(j, a.page, a.page_shift)] * a.page + wa_mod(j, a.page, a.page_shift);
     };
 
     // this wave's 16 query rows as B operands: lane (qi, g) holds Q[row qi][32 kk + 8 g .. + 8]
@@ -435,7 +440,7 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
         #pragma unroll
         for (int i = 0; i < KPT; i++) krow[i] = entry_row(k0 + (t + i * 256) / (DIM / 8));
         #pragma unroll
-        for (int i = 0; i < VPT; i++) vrow[i] = entry_row(k0 + (t + i * 256) / (VDIM / 8));
+        for (int i = 0; i < VPT; i++) vrow[i] = DIM == VDIM ? krow[i] : entry_row(k0 + (t + i * 256) / (VDIM / 8));
     };
     auto fetch = [&]() {
         #pragma unroll
@@ -609,6 +614,8 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
     }
 }
 
+static int wa_log2_exact(int x) { int sh = 0; while ((1 << sh) < x) sh++; return x > 0 && (1 << sh) == x ? sh : -1; }
+
 template <int DIM, int VDIM>
 static void wm_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
 {
@@ -657,10 +664,11 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
         if (e < NB)
         {
             const int b0 = e * a.pool;
-            return -1 - ((long long)bt[b0 / a.page] * a.per_page + (b0 % a.page) / a.pool);
+            return -1 - ((long long)bt[wa_div(b0, a.page, a.page_shift)] * a.per_page
+                         + wa_div(wa_mod(b0, a.page, a.page_shift), a.pool, a.pool_shift));
         }
         const int j = j_lo + (e - NB);
-        return (long long)bt[j / a.page] * a.page + j % a.page;
+        return (long long)bt[wa_div(j, a.page, a.page_shift)] * a.page + wa_mod(j, a.page, a.page_shift);
     };
     const int head = kh * hpg + h0 + min(qi, nh - 1);
     u32x4 qb[KK];
@@ -681,7 +689,7 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
         #pragma unroll
         for (int i = 0; i < KPT; i++) krow[i] = entry_row(k0 + (t + i * 256) / (DIM / 8));
         #pragma unroll
-        for (int i = 0; i < VPT; i++) vrow[i] = entry_row(k0 + (t + i * 256) / (VDIM / 8));
+        for (int i = 0; i < VPT; i++) vrow[i] = DIM == VDIM ? krow[i] : entry_row(k0 + (t + i * 256) / (VDIM / 8));
     };
     auto fetch = [&]() {
         #pragma unroll
@@ -900,7 +908,7 @@ extern "C" int exl2_window_attn(const void* q, const void* k_cache, const void* 
     a.q = q; a.k_cache = k_cache; a.v_cache = v_cache; a.k_pool = k_pool; a.v_pool = v_pool; a.sink = sink; a.gate = gate; a.ldg = ldg;
     a.vfreq = vfreq; a.v_rot = v_rot; a.interleaved = interleaved; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table;
     a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
-    a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window;
+    a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window; a.page_shift = a.pool_shift = -1;
     const size_t smem = (size_t)(dim + vdim) * 4;
     if (dtype == 0) LAUNCH(window_attn_kernel<u16>, dim3(rows, heads), dim3(256), smem, stream, a);
     else LAUNCH(window_attn_kernel<float>, dim3(rows, heads), dim3(256), smem, stream, a);
@@ -941,6 +949,7 @@ extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const 
     a.vfreq = vfreq; a.v_rot = v_rot; a.interleaved = interleaved; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table;
     a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
     a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window;
+    a.page_shift = wa_log2_exact(page); a.pool_shift = pool > 0 ? wa_log2_exact(pool) : -1;
     m.tile_row0 = tile_row0; m.tile_rows = tile_rows;
     hipStream_t s = (hipStream_t)stream;
     if (tile_mode == 1)

@@ -192,7 +192,7 @@ def test_chunked_scan_equals_the_recurrence(be, heads, groups, N, P):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("dim,groups", [(24, 1), (24, 3), (600, 2)])
+@pytest.mark.parametrize("dim,groups", [(24, 1), (24, 3), (600, 2), (4100, 1)])
 def test_gated_group_norm(be, dtype, dim, groups):
     rng = np.random.default_rng(dim + groups)
     rows, ldz, eps = 4, dim + 7, 1e-4
