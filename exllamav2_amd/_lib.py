@@ -126,7 +126,7 @@ PROTOTYPES = {
     "exl2_kv_rot_append": (ci, [vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, vp, cf, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]),
     "exl2_window_attn": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
     "exl2_window_attn_tiles_supported": (ci, [ci, ci]),
-    "exl2_window_attn_tiles": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
+    "exl2_window_attn_tiles": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, ci, ci, ci, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

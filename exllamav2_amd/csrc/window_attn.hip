@@ -365,6 +365,9 @@ struct WinMfmaArgs
 {
     WinAttnArgs w;
     const int* tile_row0; const int* tile_rows;
+    // decoded tokens, nsplit > 1: the steps of a row's key list are dealt to nsplit workgroups; partial results go to
+    // part_o fp32 [rows, H, nsplit, vdim] (sums relative to the partial maximum) and part_ml fp32 [rows, H, nsplit, 2] (maximum, sum)
+    float* part_o; float* part_ml; int nsplit;
 };
 
 #define WM_BK 64
@@ -649,14 +652,17 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
     const int t = tid(), lane = lane_id(), wv = wave_id();
     const int qi = lane & 15, g = lane >> 4;
     const int kh = bid_y();
-    const int hpg = a.H / a.G, h0 = bid_z() * 16, nh = min(16, hpg - h0);      // this workgroup's heads: kh * hpg + h0 .. + nh
+    const int split = bid_z() % m.nsplit;
+    const int hpg = a.H / a.G, h0 = (bid_z() / m.nsplit) * 16, nh = min(16, hpg - h0);      // this workgroup's heads: kh * hpg + h0 .. + nh
     const int r = m.tile_row0[bid_x()];
     const int pos = a.row_pos[r];
     const int* bt = a.block_table + (long long)a.row_seq[r] * a.bt_stride;
     const int NB = wa_blocks_seen(pos, a.window, a.pool);
     const int j_lo = max(0, pos - a.window + 1);
     const int total = NB + (pos - j_lo + 1);
-    const int n_steps = (total + WD_BK - 1) / WD_BK;
+    const int all_steps = (total + WD_BK - 1) / WD_BK;
+    const int per_split = (all_steps + m.nsplit - 1) / m.nsplit;
+    const int step_lo = split * per_split, n_steps = min(all_steps, step_lo + per_split);      // this workgroup's steps: step_lo .. n_steps
     const u16* kc = (const u16*)a.k_cache; const u16* vc = (const u16*)a.v_cache;
     const u16* kp = (const u16*)a.k_pool; const u16* vp = (const u16*)a.v_pool;
     auto entry_row = [&](int e) -> long long {
@@ -680,7 +686,8 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
     f32x4 ot[DB];
     #pragma unroll
     for (int d = 0; d < DB; d++) ot[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = (a.sink && wv == 0) ? a.sink[head] : WM_NEG_BIG, l_run = (a.sink && wv == 0) ? 1.0f : 0.0f;
+    const bool with_sink = a.sink && wv == 0 && split == 0;      // the sink counts once
+    float m_run = with_sink ? a.sink[head] : WM_NEG_BIG, l_run = with_sink ? 1.0f : 0.0f;
 
     long long krow[KPT], vrow[VPT];
     u32x4 kreg[KPT], vreg[VPT];
@@ -725,10 +732,13 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
     };
     static_assert(KP % 256 == 0 && VP % 256 == 0, "a step is a whole number of 16-byte pieces per thread");
 
-    lookup(0);
-    fetch();
-    if (n_steps > 1) lookup(1);
-    for (int step = 0; step < n_steps; step++)
+    if (step_lo < n_steps)
+    {
+        lookup(step_lo);
+        fetch();
+        if (step_lo + 1 < n_steps) lookup(step_lo + 1);
+    }
+    for (int step = step_lo; step < n_steps; step++)
     {
         block_sync();
         stage();
@@ -821,6 +831,14 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
             u = fmaf(s_o[(w * VDIM + ia) * 16 + q], sc2, u);
             v = fmaf(s_o[(w * VDIM + ib) * 16 + q], sc2, v);
         }
+        const int hd = kh * hpg + h0 + q;
+        if (m.nsplit > 1)                                        // partial result: the merge kernel finishes the row
+        {
+            const long long pi = ((long long)r * a.H + hd) * m.nsplit + split;
+            m.part_o[pi * VDIM + ia] = u; m.part_o[pi * VDIM + ib] = v;
+            if (pr == 0) { m.part_ml[pi * 2] = mx; m.part_ml[pi * 2 + 1] = l; }
+            continue;
+        }
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
         u *= inv; v *= inv;
         if (a.v_rot)
@@ -830,13 +848,56 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
             const float u2 = u * c + v * sn, v2 = v * c - u * sn;
             u = u2; v = v2;
         }
-        const int hd = kh * hpg + h0 + q;
         if (a.gate)
         {
             const float* gt = a.gate + (long long)r * a.ldg + hd * VDIM;
             u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib]));
         }
         u16* op = (u16*)a.out + ((long long)r * a.H + hd) * VDIM;
+        op[ia] = f32_to_bf16(u); op[ib] = f32_to_bf16(v);
+    }
+}
+
+// grid (decoded rows, heads): joins the nsplit partial results of a row's head, turns the output back, gates and stores it
+KERNEL void __launch_bounds__(64) window_attn_merge_kernel(const WinMfmaArgs m)
+{
+    const WinAttnArgs& a = m.w;
+    const int r = m.tile_row0[bid_x()], hd = bid_y();
+    const long long p0 = ((long long)r * a.H + hd) * m.nsplit;
+    float mx = WM_NEG_BIG;
+    for (int sp = 0; sp < m.nsplit; sp++) mx = fmaxf(mx, m.part_ml[(p0 + sp) * 2]);
+    float l = 0.0f;
+    for (int sp = 0; sp < m.nsplit; sp++)
+    {
+        const float ms = m.part_ml[(p0 + sp) * 2];
+        if (ms > 0.5f * WM_NEG_BIG) l = fmaf(m.part_ml[(p0 + sp) * 2 + 1], expf(ms - mx), l);
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const float fpos = (float)a.row_pos[r];
+    const float* gt = a.gate ? a.gate + (long long)r * a.ldg + hd * a.vdim : nullptr;
+    u16* op = (u16*)a.out + ((long long)r * a.H + hd) * a.vdim;
+    for (int pr = tid(); pr < a.vdim / 2; pr += 64)
+    {
+        int ia, ib;
+        wa_pair(pr, a.vdim, a.interleaved, ia, ib);
+        float u = 0.0f, v = 0.0f;
+        for (int sp = 0; sp < m.nsplit; sp++)
+        {
+            const float ms = m.part_ml[(p0 + sp) * 2];
+            if (ms <= 0.5f * WM_NEG_BIG) continue;
+            const float sc = expf(ms - mx);
+            u = fmaf(m.part_o[(p0 + sp) * a.vdim + ia], sc, u);
+            v = fmaf(m.part_o[(p0 + sp) * a.vdim + ib], sc, v);
+        }
+        u *= inv; v *= inv;
+        if (a.v_rot)
+        {
+            const float ang = fpos * a.vfreq[pr];
+            const float c = cosf(ang), sn = sinf(ang);
+            const float u2 = u * c + v * sn, v2 = v * c - u * sn;
+            u = u2; v = v2;
+        }
+        if (gt) { u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib])); }
         op[ia] = f32_to_bf16(u); op[ib] = f32_to_bf16(v);
     }
 }
@@ -851,7 +912,8 @@ static void wd_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
     if (exl2_first_on_device(attr_done))
         (void)hipFuncSetAttribute((const void*)window_attn_decode_kernel<DIM, VDIM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     const int hpg = m.w.H / m.w.G;
-    LAUNCH((window_attn_decode_kernel<DIM, VDIM>), dim3(tiles, m.w.G, (hpg + 15) / 16), dim3(256), lds, s, m);
+    LAUNCH((window_attn_decode_kernel<DIM, VDIM>), dim3(tiles, m.w.G, m.nsplit * ((hpg + 15) / 16)), dim3(256), lds, s, m);
+    if (m.nsplit > 1) LAUNCH(window_attn_merge_kernel, dim3(tiles, m.w.H), dim3(64), 0, s, m);
 }
 
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
@@ -926,13 +988,16 @@ extern "C" int exl2_window_attn_tiles_supported(int dim, int vdim)
 /* exl2_window_attn on the matrix cores (bfloat16, head sizes of exl2_window_attn_tiles_supported; gate rows and offsets multiples
    of 4 values).  The step's rows come as tiles.  tile_mode 64: tile i = rows tile_row0[i] .. + tile_rows[i], <= 64 consecutive
    positions of ONE sequence (portions of prompts; one head per workgroup).  tile_mode 1: the single rows tile_row0[i] (decoded
-   tokens; the heads of a key / value head share one pass over the keys). */
+   tokens; the heads of a key / value head share one pass over the keys); nsplit > 1 deals the key list's steps of 128 entries to
+   nsplit workgroups, part_o fp32 [rows, heads, nsplit, vdim] and part_ml fp32 [rows, heads, nsplit, 2] are scratch indexed by row. */
 extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
                                       const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
                                       const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
-                                      void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, int heads,
-                                      int kv_heads, int dim, int vdim, int window, void* stream)
+                                      void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
+                                      float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, void* stream)
 {
+    EXL2_REQUIRE(nsplit >= 1 && nsplit <= 64 && (nsplit == 1 || (tile_mode == 1 && part_o && part_ml)),
+                 "window_attn_tiles: key splits (1 .. 64) need tile_mode 1 and scratch");
     EXL2_REQUIRE(q && k_cache && v_cache && row_seq && row_pos && block_table && out && tile_row0, "window_attn_tiles: null operand");
     EXL2_REQUIRE(tile_mode == 64 || tile_mode == 1, "window_attn_tiles: tile_mode is 64 or 1");
     EXL2_REQUIRE(tile_mode == 1 || tile_rows, "window_attn_tiles: tile_rows missing");
@@ -950,7 +1015,7 @@ extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const 
     a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
     a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window;
     a.page_shift = wa_log2_exact(page); a.pool_shift = pool > 0 ? wa_log2_exact(pool) : -1;
-    m.tile_row0 = tile_row0; m.tile_rows = tile_rows;
+    m.tile_row0 = tile_row0; m.tile_rows = tile_rows; m.part_o = part_o; m.part_ml = part_ml; m.nsplit = nsplit;
     hipStream_t s = (hipStream_t)stream;
     if (tile_mode == 1)
     {

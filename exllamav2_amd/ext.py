@@ -980,7 +980,7 @@ class ExtC:
 
     def window_attn_tiles(self, q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg: int, gate_off: int, vfreq, v_rot: bool,
                           interleaved: bool, row_seq, row_pos, block_table, page: int, pool: int, out, tiles, tile_mode: int, heads: int,
-                          kv_heads: int, dim: int, vdim: int, window: int) -> None:
+                          kv_heads: int, dim: int, vdim: int, window: int, nsplit: int = 1, part_o=None, part_ml=None) -> None:
         """tile_mode 64: tiles = (tile_row0 int32 [n], tile_rows int32 [n], n), runs of <= 64 consecutive positions of one sequence;
         tile_mode 1: tiles = (rows int32 [n], None, n), single decoded rows"""
         row0, nrows, n = tiles
@@ -991,7 +991,8 @@ class ExtC:
             self._ptr(v_pool, bf, "v_pool"), self._ptr(sink, torch.float32, "sink"), gp, int(ldg), self._ptr(vfreq, torch.float32, "vfreq"),
             int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
             self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, bf, "out"),
-            self._ptr(row0, torch.int32, "tile_row0"), self._ptr(nrows, torch.int32, "tile_rows"), int(n), int(tile_mode), int(heads),
+            self._ptr(row0, torch.int32, "tile_row0"), self._ptr(nrows, torch.int32, "tile_rows"), int(n), int(tile_mode),
+            self._ptr(part_o, torch.float32, "part_o"), self._ptr(part_ml, torch.float32, "part_ml"), int(nsplit), int(heads),
             int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
 
     def graph_begin_capture(self, stream: int | None) -> None:

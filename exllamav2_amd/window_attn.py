@@ -43,6 +43,8 @@ def rotary_tables(base: float, dims: int, scaling: dict | None, device):
 
 
 class WindowAttention:
+    MAX_SPLIT = 16                                            # decoded tokens: workgroups that share one row's key list
+
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, kv_heads: int, dim: int, vdim: int, window: int, pool: int,
                  rot_base: float, rot_dims: int, rot_scaling: dict | None, scale: float, rotate_values: bool = True,
                  interleaved: bool = False):
@@ -105,7 +107,15 @@ class WindowAttention:
             if batch.tiles64 is not None:
                 ext.window_attn_tiles(*common, batch.tiles64, 64, H, G, dim, vd, self.window)
             if batch.tiles1 is not None:
-                ext.window_attn_tiles(*common, (batch.tiles1[0], None, batch.tiles1[1]), 1, H, G, dim, vd, self.window)
+                row0, n, max_pos = batch.tiles1
+                # the longest key list among the rows: window tokens + pooled blocks; its steps of 128 entries go to up to 16 workgroups
+                entries = min(self.window, max_pos + 1) + (max(0, max_pos - self.window + 1) // self.pool if self.pool else 0)
+                nsplit = max(1, min(self.MAX_SPLIT, -(-entries // 128)))
+                part_o = part_ml = None
+                if nsplit > 1:
+                    part_o = m.buf("attn.part_o", (rows, H, nsplit, vd), f32)
+                    part_ml = m.buf("attn.part_ml", (rows, H, nsplit, 2), f32)
+                ext.window_attn_tiles(*common, (row0, None, n), 1, H, G, dim, vd, self.window, nsplit=nsplit, part_o=part_o, part_ml=part_ml)
         else:
             ext.window_attn(*common, rows, H, G, dim, vd, self.window)
         return self.o.forward(o, rows, out=m.buf("mix.y", (rows, m.width), f32))

@@ -504,13 +504,15 @@ int exl2_window_attn(const void* q, const void* k_cache, const void* v_cache, co
 /* exl2_window_attn on the matrix cores: bfloat16, head sizes for which exl2_window_attn_tiles_supported returns 1 (others:
    EXL2_E_UNSUPPORTED), gate rows 16-byte aligned.  The step's rows come as tiles.  tile_mode 64: tile i = rows tile_row0[i] ..
    + tile_rows[i], at most 64 consecutive positions of ONE sequence (portions of prompts).  tile_mode 1: the single rows
-   tile_row0[i] (decoded tokens: the query heads of a key / value head share one pass over the keys). */
+   tile_row0[i] (decoded tokens: the query heads of a key / value head share one pass over the keys); nsplit > 1 deals the key
+   list's steps of 128 entries to nsplit workgroups and a second launch joins them (part_o fp32 [rows, heads, nsplit, vdim], part_ml
+   fp32 [rows, heads, nsplit, 2]: scratch indexed by row). */
 int exl2_window_attn_tiles_supported(int dim, int vdim);
 int exl2_window_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
                            const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
                            const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
-                           void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, int heads,
-                           int kv_heads, int dim, int vdim, int window, void* stream);
+                           void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
+                           float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, void* stream);
 
 #ifdef __cplusplus
 }

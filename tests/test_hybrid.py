@@ -256,7 +256,11 @@ class KernelAttention:
         if tiles:
             assert be.ext.window_attn_tiles_supported(self.dtype, dim, vd)
             if rows == 1:                                         # a decoded token: the kernel that shares the keys among a group's heads
-                be.ext.window_attn_tiles(*common, (ints(be, [0]), None, 1), 1, H, G, dim, vd, m["mask"]["size"])
+                nsplit = [1, 3, 2][pos[0] % 3]                    # (also with the key list dealt to several workgroups, some of them idle)
+                part_o = torch.zeros((1, H, nsplit, vd), dtype=F32, device=be.device)
+                part_ml = torch.zeros((1, H, nsplit, 2), dtype=F32, device=be.device)
+                be.ext.window_attn_tiles(*common, (ints(be, [0]), None, 1), 1, H, G, dim, vd, m["mask"]["size"], nsplit=nsplit,
+                                         part_o=part_o, part_ml=part_ml)
             else:
                 row0 = list(range(0, rows, 64))
                 be.ext.window_attn_tiles(*common, (ints(be, row0), ints(be, [min(64, rows - r) for r in row0]), len(row0)), 64, H, G, dim, vd,
