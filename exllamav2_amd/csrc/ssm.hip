@@ -24,7 +24,7 @@ DEV float ss_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 
 // ---- causal convolution + SiLU ------------------------------------------------------------------------------------------------
 
-#define CONV_MAX_TAPS 8
+#define CONV_MAX_TAPS 16
 #define CONV_TOKENS 32                       // consecutive rows of a span that one workgroup walks
 
 struct ConvArgs
@@ -115,7 +115,7 @@ KERNEL void __launch_bounds__(256) conv_tail_kernel(const ConvArgs a)
 // ---- selective scan -------------------------------------------------------------------------------------------------------------
 
 #define SCAN_CHUNK 16                        // tokens staged in LDS per round
-#define SCAN_MAX_NPT 64                      // state rows per thread
+#define SCAN_MAX_NPT 128                     // state rows per thread
 
 struct ScanArgs
 {
@@ -542,6 +542,7 @@ extern "C" int exl2_ssm_scan(const float* u, int ldu, const float* B, const floa
     if (npt <= 8) LAUNCH(scan_kernel<8>, grid, block, smem, stream, a);
     else if (npt <= 16) LAUNCH(scan_kernel<16>, grid, block, smem, stream, a);
     else if (npt <= 32) LAUNCH(scan_kernel<32>, grid, block, smem, stream, a);
+    else if (npt <= 64) LAUNCH(scan_kernel<64>, grid, block, smem, stream, a);
     else LAUNCH(scan_kernel<SCAN_MAX_NPT>, grid, block, smem, stream, a);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;

@@ -88,7 +88,7 @@ def spans_of(be, lens):
     return ints(be, row0), ints(be, lens), len(lens), max(lens)
 
 
-@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+@pytest.mark.parametrize("taps", [1, 2, 4, 7, 12])
 def test_causal_conv_over_spans_and_steps(be, taps):
     """two sequences in two slots fed in unequal portions (shorter and longer than the taps, one token, 40 tokens): every output
     equals the convolution over the sequence's whole history; a slot that is used again starts from zeros"""
@@ -114,7 +114,7 @@ def test_causal_conv_over_spans_and_steps(be, taps):
                 r += 1
 
 
-@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 8, 8), (3, 1, 5, 48), (2, 2, 33, 6), (1, 1, 16, 64), (6, 3, 128, 64), (2, 1, 7, 100)])
+@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 8, 8), (3, 1, 5, 48), (2, 2, 33, 6), (1, 1, 16, 64), (6, 3, 128, 64), (2, 1, 7, 100), (1, 1, 256, 128)])
 def test_selective_scan_over_spans_and_steps(be, heads, groups, N, P):
     """portions of 1 .. 37 tokens of two sequences: the state carried in the slot gives what one pass over the whole sequence gives"""
     rng = np.random.default_rng(heads * 100 + N)
