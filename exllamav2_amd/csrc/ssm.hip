@@ -227,6 +227,7 @@ struct SsdArgs
     float* zbuf;                             // [chunks of the step, heads, N, P]
     float* dbuf;                             // [chunks of the step, heads]: exp(c_L)
     const int* span_chunk0;                  // first chunk of every span
+    int nh;                                  // rows of the state the output kernel stages at a time (divides N, a multiple of 4)
 };
 
 // step sizes, log decays and their running sum for the chunk's tokens (rows past the chunk's end: zeros); thread t < SSD_L = token t
@@ -334,7 +335,13 @@ KERNEL void __launch_bounds__(256) ssd_carry_kernel(const SsdArgs g)
     *st = S;
 }
 
-KERNEL void __launch_bounds__(256) ssd_chunk_out_kernel(const SsdArgs g)
+// The state dimension goes by in slices of g.nh rows so that the staged images stay small enough for two workgroups per CU: per
+// slice the C and B columns are staged, M accumulates C . B, then the slice of the entering state takes B's place and the
+// inter-chunk product accumulates C . S.  M's 4 x 4 register tile is rows ra + 16 i x columns cb + 16 j (lanes walk consecutive
+// rows: conflict-free 16-byte LDS reads; the pairs j > i lie above the diagonal and are skipped); y tiles are 4 tokens x 4 values.
+#define SSD_YT 2                             // y tiles per thread: vdim <= 128
+
+KERNEL void __launch_bounds__(256, 2) ssd_chunk_out_kernel(const SsdArgs g)
 {
     DYN_SMEM(smem);
     const ScanArgs& a = g.s;
@@ -343,77 +350,94 @@ KERNEL void __launch_bounds__(256) ssd_chunk_out_kernel(const SsdArgs g)
     if (c * SSD_L >= n_tok) return;
     const long long row0 = a.span_row0[sp] + c * SSD_L;
     const int lc = min(SSD_L, n_tok - c * SSD_L);
-    const int N = a.N, P = a.P, grp = h / (a.heads / a.groups), t = tid();
-    const int NS = N + 4;                                        // row stride of the [token][state] images: rows fall into different banks
+    const int N = a.N, P = a.P, nh = g.nh, grp = h / (a.heads / a.groups), t = tid();
+    const int NS = nh + 4, MS = SSD_L + 4;
     float* s_dt = (float*)smem;                                  // [L]
     float* s_cum = s_dt + SSD_L;                                 // [L]
     float* s_C = s_cum + SSD_L;                                  // [L][NS]
-    float* s_BS = s_C + SSD_L * NS;                              // [L][NS] B, later [N][P] the state entering the chunk
-    float* s_X = s_BS + max(SSD_L * NS, N * P);                  // [L][P]
-    float* s_M = s_X + SSD_L * P;                                // [L][L + 4]
-    const int MS = SSD_L + 4;
+    float* s_BS = s_C + SSD_L * NS;                              // [L][NS] B, then [nh][P] the slice of the state entering the chunk
+    float* s_X = s_BS + max(SSD_L * NS, nh * P);                 // [L][P]
+    float* s_M = s_X + SSD_L * P;                                // [L][MS]
     ssd_stage_decay(a, h, row0, lc, s_dt, s_cum);
-    for (int i = t; i < SSD_L * N; i += 256)
-    {
-        const int tok = i / N, n = i % N;
-        const bool live = tok < lc;
-        s_C[tok * NS + n] = live ? a.C[(row0 + tok) * a.ldbc + grp * N + n] : 0.0f;
-        s_BS[tok * NS + n] = live ? a.B[(row0 + tok) * a.ldbc + grp * N + n] : 0.0f;
-    }
     for (int i = t; i < SSD_L * P; i += 256)
     {
         const int tok = i / P, p = i % P;
         s_X[i] = tok < lc ? a.u[(row0 + tok) * a.ldu + h * P + p] * s_dt[tok] : 0.0f;
     }
-    block_sync();
-    // M[t][s] = (C_t . B_s) exp(c_t - c_s) for s <= t, 0 above the diagonal: one 4 x 4 tile per thread
-    {
-        const int t0 = (t / (SSD_L / 4)) * 4, s0 = (t % (SSD_L / 4)) * 4;
-        float acc[4][4] = {};
-        if (s0 <= t0 + 3)
-            for (int n = 0; n < N; n += 4)
-            {
-                f32x4 cv[4], bv[4];
-                #pragma unroll
-                for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (t0 + i) * NS + n); bv[i] = *(const f32x4*)(s_BS + (s0 + i) * NS + n); }
-                #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        #pragma unroll
-                        for (int k = 0; k < 4; k++) acc[i][j] = fmaf(cv[i][k], bv[j][k], acc[i][j]);
-            }
-        #pragma unroll
-        for (int i = 0; i < 4; i++)
-            #pragma unroll
-            for (int j = 0; j < 4; j++)
-                s_M[(t0 + i) * MS + s0 + j] = s0 + j <= t0 + i ? acc[i][j] * expf(s_cum[t0 + i] - s_cum[s0 + j]) : 0.0f;
-    }
-    block_sync();                                                // B is no longer needed: its place takes the entering state
-    {
-        const float* zin = g.zbuf + ((long long)(g.span_chunk0[sp] + c) * a.heads + h) * (long long)N * P;
-        for (int i = t * 4; i < N * P; i += 1024) *(f32x4*)(s_BS + i) = *(const f32x4*)(zin + i);
-    }
-    block_sync();
-    const float Dh = a.D[h];
+    const int ra = t / 16, cb = t % 16;
     const int tp = P / 4, tiles = (SSD_L / 4) * tp;
-    for (int tile = t; tile < tiles; tile += 256)
+    const float* zin = g.zbuf + ((long long)(g.span_chunk0[sp] + c) * a.heads + h) * (long long)N * P;
+    float macc[4][4] = {};
+    float inter[SSD_YT][4][4] = {};
+    for (int n0 = 0; n0 < N; n0 += nh)
     {
-        const int t0 = (tile / tp) * 4, p0 = (tile % tp) * 4;
-        if (t0 >= lc) continue;
-        float inter[4][4] = {}, intra[4][4] = {};
-        for (int n = 0; n < N; n += 4)
+        block_sync();                                            // the previous slice's readers are done
+        for (int i = t; i < SSD_L * nh; i += 256)
         {
-            f32x4 cv[4], sv[4];
+            const int tok = i / nh, n = i % nh;
+            const bool live = tok < lc;
+            s_C[tok * NS + n] = live ? a.C[(row0 + tok) * a.ldbc + grp * N + n0 + n] : 0.0f;
+            s_BS[tok * NS + n] = live ? a.B[(row0 + tok) * a.ldbc + grp * N + n0 + n] : 0.0f;
+        }
+        block_sync();
+        for (int n = 0; n < nh; n += 4)
+        {
+            f32x4 cv[4], bv[4];
             #pragma unroll
-            for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (t0 + i) * NS + n); sv[i] = *(const f32x4*)(s_BS + (n + i) * P + p0); }
+            for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (ra + 16 * i) * NS + n); bv[i] = *(const f32x4*)(s_BS + (cb + 16 * i) * NS + n); }
             #pragma unroll
             for (int i = 0; i < 4; i++)
                 #pragma unroll
-                for (int k = 0; k < 4; k++)
-                    #pragma unroll
-                    for (int j = 0; j < 4; j++) inter[i][j] = fmaf(cv[i][k], sv[k][j], inter[i][j]);
+                for (int j = 0; j < 4; j++)
+                    if (j <= i)
+                    {
+                        #pragma unroll
+                        for (int k = 0; k < 4; k++) macc[i][j] = fmaf(cv[i][k], bv[j][k], macc[i][j]);
+                    }
         }
+        block_sync();                                            // B is no longer needed: its place takes the state's slice
+        for (int i = t * 4; i < nh * P; i += 1024) *(f32x4*)(s_BS + i) = *(const f32x4*)(zin + (long long)n0 * P + i);
+        block_sync();
+        #pragma unroll
+        for (int yt = 0; yt < SSD_YT; yt++)
+        {
+            const int tile = t + 256 * yt;
+            if (tile >= tiles) break;
+            const int t0 = (tile / tp) * 4, p0 = (tile % tp) * 4;
+            if (t0 >= lc) continue;
+            for (int n = 0; n < nh; n += 4)
+            {
+                f32x4 cv[4], sv[4];
+                #pragma unroll
+                for (int i = 0; i < 4; i++) { cv[i] = *(const f32x4*)(s_C + (t0 + i) * NS + n); sv[i] = *(const f32x4*)(s_BS + (n + i) * P + p0); }
+                #pragma unroll
+                for (int i = 0; i < 4; i++)
+                    #pragma unroll
+                    for (int k = 0; k < 4; k++)
+                        #pragma unroll
+                        for (int j = 0; j < 4; j++) inter[yt][i][j] = fmaf(cv[i][k], sv[k][j], inter[yt][i][j]);
+            }
+        }
+    }
+    // M[t][s] = (C_t . B_s) exp(c_t - c_s) for s <= t, 0 above the diagonal
+    #pragma unroll
+    for (int i = 0; i < 4; i++)
+        #pragma unroll
+        for (int j = 0; j < 4; j++)
+        {
+            const int tt = ra + 16 * i, ss = cb + 16 * j;
+            s_M[tt * MS + ss] = ss <= tt ? macc[i][j] * expf(s_cum[tt] - s_cum[ss]) : 0.0f;
+        }
+    block_sync();
+    const float Dh = a.D[h];
+    #pragma unroll
+    for (int yt = 0; yt < SSD_YT; yt++)
+    {
+        const int tile = t + 256 * yt;
+        if (tile >= tiles) break;
+        const int t0 = (tile / tp) * 4, p0 = (tile % tp) * 4;
+        if (t0 >= lc) continue;
+        float intra[4][4] = {};
         for (int s0 = 0; s0 <= t0; s0 += 4)
         {
             f32x4 mv[4], xv[4];
@@ -434,7 +458,7 @@ KERNEL void __launch_bounds__(256) ssd_chunk_out_kernel(const SsdArgs g)
             const f32x4 uv = *(const f32x4*)(a.u + (row0 + t0 + i) * a.ldu + h * P + p0);
             f32x4 y;
             #pragma unroll
-            for (int j = 0; j < 4; j++) y[j] = fmaf(e, inter[i][j], intra[i][j]) + Dh * uv[j];
+            for (int j = 0; j < 4; j++) y[j] = fmaf(e, inter[yt][i][j], intra[i][j]) + Dh * uv[j];
             *(f32x4*)(a.y + (row0 + t0 + i) * a.ldy + h * P + p0) = y;
         }
     }
@@ -548,16 +572,33 @@ extern "C" int exl2_ssm_scan(const float* u, int ldu, const float* B, const floa
     return EXL2_OK;
 }
 
-static size_t ssd_out_smem(int N, int P)
+static size_t ssd_out_smem(int nh, int P)
 {
-    const size_t bs = (size_t)SSD_L * (N + 4) > (size_t)N * P ? (size_t)SSD_L * (N + 4) : (size_t)N * P;
-    return sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (N + 4) + bs + (size_t)SSD_L * P + (size_t)SSD_L * (SSD_L + 4));
+    const size_t bs = (size_t)SSD_L * (nh + 4) > (size_t)nh * P ? (size_t)SSD_L * (nh + 4) : (size_t)nh * P;
+    return sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (nh + 4) + bs + (size_t)SSD_L * P + (size_t)SSD_L * (SSD_L + 4));
+}
+
+// the slice of the state dimension the output kernel stages: the largest N / {1, 2, 4, 8} (a multiple of 4) whose images let two
+// workgroups share a CU's LDS, else the smallest that fits at all; 0: none fits
+static int ssd_slice(int N, int P)
+{
+    int fits = 0;
+    for (int parts = 1; parts <= 8; parts *= 2)
+    {
+        if (N % (4 * parts) != 0) break;
+        const int nh = N / parts;
+        const size_t sm = ssd_out_smem(nh, P);
+        if (sm <= 76 * 1024) return nh;
+        if (sm <= 160 * 1024 - 256) fits = nh;
+    }
+    return fits;
 }
 
 /* 1 if exl2_ssm_scan_chunked takes this shape (sizes in fours that fit the LDS), 0 otherwise */
 extern "C" int exl2_ssm_scan_chunked_supported(int n_state, int vdim)
 {
-    return n_state > 0 && vdim > 0 && n_state % 4 == 0 && vdim % 4 == 0 && ssd_out_smem(n_state, vdim) <= 160 * 1024 - 256;
+    return n_state > 0 && vdim > 0 && n_state % 4 == 0 && vdim % 4 == 0 && vdim <= 64 * SSD_YT && ssd_slice(n_state, vdim) > 0
+           && sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (n_state + vdim)) <= 160 * 1024 - 256;
 }
 
 extern "C" int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
@@ -579,8 +620,8 @@ extern "C" int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, co
     a.u = u; a.ldu = ldu; a.B = B; a.C = C; a.ldbc = ldbc; a.dt = dt; a.lddt = lddt; a.dt_bias = dt_bias; a.A_log = A_log; a.D = D;
     a.y = y; a.ldy = ldy; a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
     a.heads = heads; a.groups = groups; a.N = n_state; a.P = vdim; a.KS = 0;
-    g.zbuf = zbuf; g.dbuf = dbuf; g.span_chunk0 = span_chunk0;
-    const size_t smem1 = sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (n_state + vdim)), smem3 = ssd_out_smem(n_state, vdim);
+    g.zbuf = zbuf; g.dbuf = dbuf; g.span_chunk0 = span_chunk0; g.nh = ssd_slice(n_state, vdim);
+    const size_t smem1 = sizeof(float) * (2 * SSD_L + (size_t)SSD_L * (n_state + vdim)), smem3 = ssd_out_smem(g.nh, vdim);
     static bool attr_done[EXL2_MAX_DEVICES];
     if (exl2_first_on_device(attr_done))
     {

@@ -148,7 +148,7 @@ def test_selective_scan_over_spans_and_steps(be, heads, groups, N, P):
     assert close(be.n(state)[2], S[2], 2e-5) and (be.n(state)[1] == 5.0).all()
 
 
-@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 8, 8), (2, 1, 128, 64), (3, 3, 12, 100), (1, 1, 32, 48)])
+@pytest.mark.parametrize("heads,groups,N,P", [(4, 2, 8, 8), (2, 1, 128, 64), (3, 3, 12, 100), (1, 1, 32, 48), (1, 1, 256, 128)])
 def test_chunked_scan_equals_the_recurrence(be, heads, groups, N, P):
     """portions of 1 .. 200 tokens (several chunks, chunks that end early) through the chunked form, mixed with the token-by-token form
     on the same slots: outputs and carried state equal the plain recurrence"""
