@@ -266,15 +266,23 @@ KERNEL void __launch_bounds__(256) ssd_chunk_state_kernel(const SsdArgs g)
     float* s_X = s_B + SSD_L * N;                                // [L][P]: d_s u_s
     ssd_stage_decay(a, h, row0, lc, s_dt, s_cum);
     const float c_end = s_cum[SSD_L - 1];
-    for (int i = t; i < SSD_L * N; i += 256)
+    // (16-byte loads, four in flight per thread: the staging loops are latency-bound otherwise)
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    #pragma unroll 4
+    for (int i = t; i < SSD_L * N / 4; i += 256)
     {
-        const int tok = i / N, n = i % N;
-        s_B[i] = tok < lc ? a.B[(row0 + tok) * a.ldbc + grp * N + n] * expf(c_end - s_cum[tok]) : 0.0f;
+        const int tok = i / (N / 4), n = (i % (N / 4)) * 4;
+        const f32x4 b = tok < lc ? *(const f32x4*)(a.B + (row0 + tok) * a.ldbc + grp * N + n) : zero4;
+        const float w = expf(c_end - s_cum[tok]);
+        *(f32x4*)(s_B + tok * N + n) = (f32x4){b[0] * w, b[1] * w, b[2] * w, b[3] * w};
     }
-    for (int i = t; i < SSD_L * P; i += 256)
+    #pragma unroll 4
+    for (int i = t; i < SSD_L * P / 4; i += 256)
     {
-        const int tok = i / P, p = i % P;
-        s_X[i] = tok < lc ? a.u[(row0 + tok) * a.ldu + h * P + p] * s_dt[tok] : 0.0f;
+        const int tok = i / (P / 4), p = (i % (P / 4)) * 4;
+        const f32x4 x = tok < lc ? *(const f32x4*)(a.u + (row0 + tok) * a.ldu + h * P + p) : zero4;
+        const float d = s_dt[tok];
+        *(f32x4*)(s_X + tok * P + p) = (f32x4){x[0] * d, x[1] * d, x[2] * d, x[3] * d};
     }
     block_sync();
     float* z = g.zbuf + ((long long)(g.span_chunk0[sp] + c) * a.heads + h) * (long long)N * P;
@@ -359,10 +367,14 @@ KERNEL void __launch_bounds__(256, 2) ssd_chunk_out_kernel(const SsdArgs g)
     float* s_X = s_BS + max(SSD_L * NS, nh * P);                 // [L][P]
     float* s_M = s_X + SSD_L * P;                                // [L][MS]
     ssd_stage_decay(a, h, row0, lc, s_dt, s_cum);
-    for (int i = t; i < SSD_L * P; i += 256)
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    #pragma unroll 4
+    for (int i = t; i < SSD_L * P / 4; i += 256)
     {
-        const int tok = i / P, p = i % P;
-        s_X[i] = tok < lc ? a.u[(row0 + tok) * a.ldu + h * P + p] * s_dt[tok] : 0.0f;
+        const int tok = i / (P / 4), p = (i % (P / 4)) * 4;
+        const f32x4 x = tok < lc ? *(const f32x4*)(a.u + (row0 + tok) * a.ldu + h * P + p) : zero4;
+        const float d = s_dt[tok];
+        *(f32x4*)(s_X + tok * P + p) = (f32x4){x[0] * d, x[1] * d, x[2] * d, x[3] * d};
     }
     const int ra = t / 16, cb = t % 16;
     const int tp = P / 4, tiles = (SSD_L / 4) * tp;
@@ -372,12 +384,13 @@ KERNEL void __launch_bounds__(256, 2) ssd_chunk_out_kernel(const SsdArgs g)
     for (int n0 = 0; n0 < N; n0 += nh)
     {
         block_sync();                                            // the previous slice's readers are done
-        for (int i = t; i < SSD_L * nh; i += 256)
+        #pragma unroll 4
+        for (int i = t; i < SSD_L * nh / 4; i += 256)
         {
-            const int tok = i / nh, n = i % nh;
+            const int tok = i / (nh / 4), n = (i % (nh / 4)) * 4;
             const bool live = tok < lc;
-            s_C[tok * NS + n] = live ? a.C[(row0 + tok) * a.ldbc + grp * N + n0 + n] : 0.0f;
-            s_BS[tok * NS + n] = live ? a.B[(row0 + tok) * a.ldbc + grp * N + n0 + n] : 0.0f;
+            *(f32x4*)(s_C + tok * NS + n) = live ? *(const f32x4*)(a.C + (row0 + tok) * a.ldbc + grp * N + n0 + n) : zero4;
+            *(f32x4*)(s_BS + tok * NS + n) = live ? *(const f32x4*)(a.B + (row0 + tok) * a.ldbc + grp * N + n0 + n) : zero4;
         }
         block_sync();
         for (int n = 0; n < nh; n += 4)
@@ -396,6 +409,7 @@ KERNEL void __launch_bounds__(256, 2) ssd_chunk_out_kernel(const SsdArgs g)
                     }
         }
         block_sync();                                            // B is no longer needed: its place takes the state's slice
+        #pragma unroll 4
         for (int i = t * 4; i < nh * P; i += 1024) *(f32x4*)(s_BS + i) = *(const f32x4*)(zin + (long long)n0 * P + i);
         block_sync();
         #pragma unroll
@@ -612,8 +626,9 @@ extern "C" int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, co
     EXL2_REQUIRE(chunk == SSD_L, "ssm_scan_chunked: chunks of %d rows (the span table was made for %d)", SSD_L, chunk);
     EXL2_REQUIRE(heads > 0 && groups > 0 && heads % groups == 0, "ssm_scan_chunked: %d heads in %d groups", heads, groups);
     EXL2_REQUIRE(exl2_ssm_scan_chunked_supported(n_state, vdim), "ssm_scan_chunked: state %d x %d outside the chunked form", n_state, vdim);
-    EXL2_REQUIRE(ldu % 4 == 0 && ldy % 4 == 0 && ((uintptr_t)u % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)zbuf % 16) == 0,
-                 "ssm_scan_chunked: rows of u / y must be 16-byte aligned");
+    EXL2_REQUIRE(ldu % 4 == 0 && ldy % 4 == 0 && ldbc % 4 == 0 && ((uintptr_t)u % 16) == 0 && ((uintptr_t)y % 16) == 0
+                 && ((uintptr_t)B % 16) == 0 && ((uintptr_t)C % 16) == 0 && ((uintptr_t)zbuf % 16) == 0,
+                 "ssm_scan_chunked: rows of u / B / C / y must be 16-byte aligned");
     if (spans <= 0 || max_span_rows <= 0) return EXL2_OK;
     SsdArgs g;
     ScanArgs& a = g.s;

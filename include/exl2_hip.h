@@ -469,7 +469,7 @@ int exl2_ssm_scan(const float* u, int ldu, const float* B, const float* C, int l
 /* exl2_ssm_scan for portions of prompts: the recurrence unrolled in chunks of `chunk` (64) rows, every (chunk, head) independent
    work around a short carry over each span's chunks.  span_chunk0[i] = number of chunks of the spans before i; zbuf fp32
    [all chunks, heads, n_state, vdim] and dbuf fp32 [all chunks, heads] are scratch.  n_state and vdim multiples of 4 that fit the
-   LDS (exl2_ssm_scan_chunked_supported), rows of u / y 16-byte aligned. */
+   LDS (exl2_ssm_scan_chunked_supported), rows of u / B / C / y 16-byte aligned. */
 int exl2_ssm_scan_chunked_supported(int n_state, int vdim);
 int exl2_ssm_scan_chunked(const float* u, int ldu, const float* B, const float* C, int ldbc, const float* dt, int lddt,
                           const float* dt_bias, const float* A_log, const float* D, float* y, int ldy, float* state,
