@@ -182,8 +182,8 @@ def hybrid_config(s: dict) -> dict:
             layers.append({"type": "attention", "mlp": None,
                            "mixer": {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"],
                                      "mask": {"pool": s["pool"], "size": s["window"]}, "scale": s["dim"] ** -0.5,
-                                     "rot": {"base": 1e6, "dims": s["rot_dims"],
-                                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}})
+                                     "rot": {"base": 500000.0, "dims": s["rot_dims"],
+                                             "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}})
     return {"architecture": "Tibalorn", "embedding": {"scale": 1.0}, "layers": layers, "logit_softcap": 30.0, "norm": {"eps": 1e-5},
             "vocab": s["vocab"], "width": s["width"]}
 

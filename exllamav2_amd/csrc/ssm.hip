@@ -68,12 +68,18 @@ KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
         }
     }
     const int t1 = min(n, t0 + CONV_TOKENS);
-    for (int t = t0; t < t1; t++)
+    float xin[CONV_TOKENS];                                      // all of the walk's inputs leave together
+    #pragma unroll
+    for (int i = 0; i < CONV_TOKENS; i++) xin[i] = t0 + i < t1 ? a.in[(long long)(r0 + t0 + i) * a.ld + c] : 0.0f;
+    #pragma unroll
+    for (int i = 0; i < CONV_TOKENS; i++)
     {
+        const int t = t0 + i;
+        if (t >= t1) break;
         #pragma unroll
         for (int k = 0; k < CONV_MAX_TAPS - 1; k++) win[k] = win[k + 1];
         // after the shift the newest value belongs at index taps - 1
-        const float cur = a.in[(long long)(r0 + t) * a.ld + c];
+        const float cur = xin[i];
         float acc = bias;
         #pragma unroll
         for (int k = 0; k < CONV_MAX_TAPS; k++)

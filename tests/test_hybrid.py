@@ -321,7 +321,7 @@ def test_attention_kernels_against_the_oracle(be, dtype, shape):
 @pytest.mark.parametrize("shape", [dict(heads=4, kv_heads=2, dim=32, vdim=32, size=40, pool=8, dims=16, page=16),
                                    dict(heads=2, kv_heads=1, dim=64, vdim=64, size=70, pool=16, dims=64, page=64, scaling=None),
                                    dict(heads=3, kv_heads=3, dim=128, vdim=64, size=33, pool=5, dims=32, page=7),
-                                   dict(heads=2, kv_heads=2, dim=96, vdim=96, size=200, pool=64, dims=24, page=256),
+                                   dict(heads=2, kv_heads=2, dim=96, vdim=96, size=200, pool=64, dims=32, page=256),
                                    dict(heads=2, kv_heads=1, dim=64, vdim=128, size=1, pool=1, dims=2, page=3),
                                    dict(heads=34, kv_heads=2, dim=32, vdim=32, size=20, pool=6, dims=8, page=32)])
 def test_matrix_core_attention_against_the_oracle(be, shape):
