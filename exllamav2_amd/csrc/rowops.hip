@@ -9,6 +9,7 @@
 // Element type T of weights / operand copies: u16 = bfloat16 bits, float.
 #include "hw.h"
 #include "errors.h"
+#include <stdint.h>
 
 template <typename T> DEV float ro_ld(const T* p);
 template <> DEV float ro_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
@@ -153,6 +154,75 @@ KERNEL void __launch_bounds__(256) add_layer_norm_kernel(const LayerNormArgs a)
     {
         const float o = (v[i] - mean) * rinv * ro_ld<T>((const T*)a.w + i) + (a.b ? ro_ld<T>((const T*)a.b + i) : 0.0f);
         if (a.out_f32) ((float*)a.out)[(long long)r * a.width + i] = o; else ro_st<T>((T*)a.out + (long long)r * a.width + i, o);
+    }
+}
+
+// The same step for rows of up to 256 * 4 * LN_VPT values in fours: a thread keeps its values in registers between the passes (no
+// LDS image), all its 16-byte loads leave together, results go out as 16-byte (fp32) or 8-byte (bfloat16) stores.
+#define LN_VPT 4
+
+template <typename T> DEV f32x4 ro_ld4(const T* p);
+template <> DEV f32x4 ro_ld4<float>(const float* p) { return *(const f32x4*)p; }
+template <> DEV f32x4 ro_ld4<u16>(const u16* p)
+{
+    const u32x2 v = *(const u32x2*)p;
+    return (f32x4){as_f32(v[0] << 16), as_f32(v[0] & 0xffff0000u), as_f32(v[1] << 16), as_f32(v[1] & 0xffff0000u)};
+}
+
+template <typename T>
+KERNEL void __launch_bounds__(256) add_layer_norm_vec_kernel(const LayerNormArgs a)
+{
+    SHARED float part[4];
+    const int r = bid_x();
+    const long long src = a.row_idx ? a.row_idx[r] : r;
+    const int nvec = a.width / 4;
+    f32x4* xr = (f32x4*)(a.x + src * a.width);
+    const f32x4* yr = a.y ? (const f32x4*)(a.y + src * a.width) : nullptr;
+    f32x4 v[LN_VPT], yv[LN_VPT];
+    #pragma unroll
+    for (int e = 0; e < LN_VPT; e++)
+    {
+        const int i = tid() + 256 * e;
+        v[e] = i < nvec ? xr[i] : (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        yv[e] = (yr && i < nvec) ? yr[i] : (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    float s = 0.0f;
+    #pragma unroll
+    for (int e = 0; e < LN_VPT; e++)
+    {
+        const int i = tid() + 256 * e;
+        if (yr)
+        {
+            v[e][0] += yv[e][0]; v[e][1] += yv[e][1]; v[e][2] += yv[e][2]; v[e][3] += yv[e][3];
+            if (i < nvec) xr[i] = v[e];
+        }
+        s += (v[e][0] + v[e][1]) + (v[e][2] + v[e][3]);
+    }
+    if (!a.w) return;
+    const float mean = block_sum_256(s, part) / (float)a.width;
+    float ss = 0.0f;
+    #pragma unroll
+    for (int e = 0; e < LN_VPT; e++)
+    {
+        if (tid() + 256 * e >= nvec) break;
+        #pragma unroll
+        for (int k = 0; k < 4; k++) { const float d = v[e][k] - mean; ss = fmaf(d, d, ss); }
+    }
+    ss = block_sum_256(ss, part);
+    const float rinv = 1.0f / sqrtf(ss / (float)a.width + a.eps);
+    #pragma unroll
+    for (int e = 0; e < LN_VPT; e++)
+    {
+        const int i = tid() + 256 * e;
+        if (i >= nvec) break;
+        const f32x4 wv = ro_ld4<T>((const T*)a.w + 4 * i);
+        const f32x4 bv = a.b ? ro_ld4<T>((const T*)a.b + 4 * i) : (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        f32x4 o;
+        #pragma unroll
+        for (int k = 0; k < 4; k++) o[k] = (v[e][k] - mean) * rinv * wv[k] + bv[k];
+        if (a.out_f32) *(f32x4*)((float*)a.out + (long long)r * a.width + 4 * i) = o;
+        else *(u32x2*)((u16*)a.out + (long long)r * a.width + 4 * i) =
+                 (u32x2){(u32)f32_to_bf16(o[0]) | ((u32)f32_to_bf16(o[1]) << 16), (u32)f32_to_bf16(o[2]) | ((u32)f32_to_bf16(o[3]) << 16)};
     }
 }
 
@@ -325,6 +395,15 @@ extern "C" int exl2_add_layer_norm(float* x, const float* y, const void* w, cons
     if (rows <= 0) return EXL2_OK;
     LayerNormArgs a;
     a.x = x; a.y = y; a.w = w; a.b = b; a.out = out; a.out_f32 = out_f32 || dtype == 1; a.row_idx = row_idx; a.width = width; a.eps = eps;
+    const bool aligned = ((uintptr_t)x % 16) == 0 && (!y || ((uintptr_t)y % 16) == 0) && (!w || ((uintptr_t)w % 16) == 0)
+                         && (!b || ((uintptr_t)b % 16) == 0) && (!out || ((uintptr_t)out % 16) == 0);
+    if (width % 4 == 0 && width <= 256 * 4 * LN_VPT && aligned)
+    {
+        if (dtype == 0) LAUNCH(add_layer_norm_vec_kernel<u16>, dim3(rows), dim3(256), 0, stream, a);
+        else LAUNCH(add_layer_norm_vec_kernel<float>, dim3(rows), dim3(256), 0, stream, a);
+        HIP_TRY(hipGetLastError());
+        return EXL2_OK;
+    }
     const size_t smem = (size_t)width * 4;
     if (smem > 48 * 1024)
     {

@@ -42,7 +42,7 @@ def close(got, want, tol):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("width", [6, 50, 300])
+@pytest.mark.parametrize("width", [6, 50, 300, 2048, 4100])
 def test_add_layer_norm(be, dtype, width):
     rng = np.random.default_rng(width)
     rows, eps = 5, 1e-3
