@@ -37,10 +37,11 @@ struct ConvArgs
     int channels, taps;
 };
 
-// grid (channel blocks, token chunks, spans): thread = one channel over CONV_TOKENS consecutive rows, the window of the last
-// taps inputs slides through registers.  Inputs in front of the span come from the slot's tail, inputs in front of the
-// sequence are zero.
-template <typename T>
+// grid (channel blocks, token chunks, spans): thread = one channel over CONV_TOKENS consecutive rows of a span; the window of the
+// last taps inputs slides through registers (MAXT of them: the smallest of 4 / 8 / 16 that holds the taps) and all of the walk's
+// inputs are requested before the first is used.  Inputs in front of the span come from the slot's tail, inputs in front of the
+// sequence are zero.  (Four channels per thread with 16-byte accesses measured slower: 120 against 74 us at 2048 x 4352.)
+template <typename T, int MAXT>
 KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
 {
     const int c = bid_x() * 256 + tid();
@@ -51,43 +52,41 @@ KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
     const int r0 = a.span_row0[sp];
     const int pos0 = a.row_pos[r0];
     const float* tail = a.tail + (long long)a.row_seq[r0] * (a.taps - 1) * a.channels;
-    float w[CONV_MAX_TAPS], win[CONV_MAX_TAPS];
+    const int t1 = min(n, t0 + CONV_TOKENS);
+    float xin[CONV_TOKENS];
     #pragma unroll
-    for (int k = 0; k < CONV_MAX_TAPS; k++) w[k] = k < a.taps ? ss_ld<T>((const T*)a.w + (long long)c * a.taps + k) : 0.0f;
+    for (int i = 0; i < CONV_TOKENS; i++) xin[i] = t0 + i < t1 ? a.in[(long long)(r0 + t0 + i) * a.ld + c] : 0.0f;
+    float w[MAXT], win[MAXT];
+    #pragma unroll
+    for (int k = 0; k < MAXT; k++) w[k] = k < a.taps ? ss_ld<T>((const T*)a.w + (long long)c * a.taps + k) : 0.0f;
     const float bias = a.bias ? ss_ld<T>((const T*)a.bias + c) : 0.0f;
-    // win[k] = input at token t - (taps - 1) + k; tokens are counted within the span, token -d is position pos0 - d
+    // win[k] = input at token t - (taps - 1) + k; before the first shift slot k holds token t0 - (taps - 1) + (k - 1); tokens are
+    // counted within the span, token -d is position pos0 - d
     #pragma unroll
-    for (int k = 0; k < CONV_MAX_TAPS; k++)
+    for (int k = 0; k < MAXT; k++)
     {
         win[k] = 0.0f;
-        if (k >= 1 && k < a.taps)                                  // slot k of the next window = token t0 - (taps - 1) + (k - 1) + ... set below
+        if (k >= 1 && k < a.taps)
         {
             const int tok = t0 - (a.taps - 1) + (k - 1);
             if (tok >= 0) win[k] = a.in[(long long)(r0 + tok) * a.ld + c];
             else if (pos0 + tok >= 0) win[k] = tail[(long long)(a.taps - 1 + tok) * a.channels + c];
         }
     }
-    const int t1 = min(n, t0 + CONV_TOKENS);
-    float xin[CONV_TOKENS];                                      // all of the walk's inputs leave together
-    #pragma unroll
-    for (int i = 0; i < CONV_TOKENS; i++) xin[i] = t0 + i < t1 ? a.in[(long long)(r0 + t0 + i) * a.ld + c] : 0.0f;
     #pragma unroll
     for (int i = 0; i < CONV_TOKENS; i++)
     {
-        const int t = t0 + i;
-        if (t >= t1) break;
+        if (t0 + i >= t1) break;
         #pragma unroll
-        for (int k = 0; k < CONV_MAX_TAPS - 1; k++) win[k] = win[k + 1];
-        // after the shift the newest value belongs at index taps - 1
-        const float cur = xin[i];
+        for (int k = 0; k < MAXT - 1; k++) win[k] = win[k + 1];
         float acc = bias;
         #pragma unroll
-        for (int k = 0; k < CONV_MAX_TAPS; k++)
+        for (int k = 0; k < MAXT; k++)
         {
-            if (k == a.taps - 1) win[k] = cur;
+            if (k == a.taps - 1) win[k] = xin[i];                // after the shift the newest value belongs at index taps - 1
             if (k < a.taps) acc = fmaf(w[k], win[k], acc);
         }
-        a.out[(long long)(r0 + t) * a.ldo + c] = ss_silu(acc);
+        a.out[(long long)(r0 + t0 + i) * a.ldo + c] = ss_silu(acc);
     }
 }
 
@@ -554,8 +553,18 @@ extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const
     a.in = in; a.ld = ld; a.w = w; a.bias = bias; a.out = out; a.ldo = ldo; a.tail = tail; a.span_row0 = span_row0; a.span_rows = span_rows;
     a.row_seq = row_seq; a.row_pos = row_pos; a.channels = channels; a.taps = taps;
     const dim3 grid((channels + 255) / 256, (max_span_rows + CONV_TOKENS - 1) / CONV_TOKENS, spans);
-    if (dtype == 0) LAUNCH(conv_silu_kernel<u16>, grid, dim3(256), 0, stream, a);
-    else LAUNCH(conv_silu_kernel<float>, grid, dim3(256), 0, stream, a);
+    if (dtype == 0)
+    {
+        if (taps <= 4) LAUNCH((conv_silu_kernel<u16, 4>), grid, dim3(256), 0, stream, a);
+        else if (taps <= 8) LAUNCH((conv_silu_kernel<u16, 8>), grid, dim3(256), 0, stream, a);
+        else LAUNCH((conv_silu_kernel<u16, CONV_MAX_TAPS>), grid, dim3(256), 0, stream, a);
+    }
+    else
+    {
+        if (taps <= 4) LAUNCH((conv_silu_kernel<float, 4>), grid, dim3(256), 0, stream, a);
+        else if (taps <= 8) LAUNCH((conv_silu_kernel<float, 8>), grid, dim3(256), 0, stream, a);
+        else LAUNCH((conv_silu_kernel<float, CONV_MAX_TAPS>), grid, dim3(256), 0, stream, a);
+    }
     if (taps > 1) LAUNCH(conv_tail_kernel, dim3((channels + 255) / 256, spans), dim3(256), 0, stream, a);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;

@@ -350,7 +350,7 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
 }
 
 // ---- bfloat16 on the matrix cores ---------------------------------------------------------------------------------------------------
-// Workgroup = one tile of <= 64 consecutive positions of one sequence x one head; wave w owns the 16 query rows 16 w .. 16 w + 15.
+// Workgroup = one tile of <= 64 RPW consecutive positions of one sequence x one head; wave w owns RPW blocks of 16 query rows.
 // The tile's key list is [pooled blocks 0 .. NB) | tokens j_lo .. last position], NB and j_lo taken for the tile as a whole and
 // masked per query row; it goes by in steps of 64 entries whose key and value rows are staged row-major in LDS (each entry's row is
 // looked up through the block table -- pooled rows in the pooled tensors -- one step ahead of its loads, two steps ahead of its use).
@@ -375,7 +375,7 @@ struct WinMfmaArgs
 
 DEV u32 wm_pack2(float lo, float hi) { return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16); }
 
-template <int DIM, int VDIM>
+template <int DIM, int VDIM, int RPW>
 KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs m)
 {
     DYN_SMEM(smem);
@@ -414,27 +414,36 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
         return (long long)bt[wa_div(j, a.page, a.page_shift)] * a.page + wa_mod(j, a.page, a.page_shift);
     };
 
-    // this wave's 16 query rows as B operands: lane (qi, g) holds Q[row qi][32 kk + 8 g .. + 8]
-    const int my_row = wv * 16 + qi;
-    const int qrow = r0 + min(my_row, n_rows - 1);
-    const int qpos = p0 + min(my_row, n_rows - 1);
-    const bool wave_live = wv * 16 < n_rows;
-    u32x4 qb[KK];
+    // this wave's RPW x 16 query rows as B operands: lane (qi, g) holds Q[row 16 n + qi][32 kk + 8 g .. + 8] of block n; every key
+    // and value fragment read from LDS feeds RPW products
+    int my_row[RPW], qrow[RPW], qpos[RPW], my_nb[RPW], my_lo[RPW];
+    u32x4 qb[RPW][KK];
+    #pragma unroll
+    for (int n = 0; n < RPW; n++)
     {
-        const u16* qp = (const u16*)a.q + ((long long)qrow * a.H + h) * DIM + 8 * g;
+        my_row[n] = (wv * RPW + n) * 16 + qi;
+        qrow[n] = r0 + min(my_row[n], n_rows - 1);
+        qpos[n] = p0 + min(my_row[n], n_rows - 1);
+        const u16* qp = (const u16*)a.q + ((long long)qrow[n] * a.H + h) * DIM + 8 * g;
         #pragma unroll
-        for (int kk = 0; kk < KK; kk++) qb[kk] = *(const u32x4*)(qp + 32 * kk);
+        for (int kk = 0; kk < KK; kk++) qb[n][kk] = *(const u32x4*)(qp + 32 * kk);
+        my_nb[n] = wa_blocks_seen(qpos[n], a.window, a.pool);
+        my_lo[n] = qpos[n] - a.window + 1;                      // first token this query sees (may be negative)
     }
-    const int my_nb = wa_blocks_seen(qpos, a.window, a.pool);
-    const int my_lo = qpos - a.window + 1;                      // first token this query sees (may be negative)
+    const bool wave_live = wv * RPW * 16 < n_rows;
     // what the wave as a whole can see: blocks below wave_nb, tokens wave_lo .. wave_hi
-    const int wp0 = p0 + min(wv * 16, n_rows - 1), wp1 = p0 + min(wv * 16 + 15, n_rows - 1);
+    const int wp0 = p0 + min(wv * RPW * 16, n_rows - 1), wp1 = p0 + min(wv * RPW * 16 + RPW * 16 - 1, n_rows - 1);
     const int wave_nb = wa_blocks_seen(wp1, a.window, a.pool), wave_lo = wp0 - a.window + 1, wave_hi = wp1;
 
-    f32x4 ot[DB];
+    f32x4 ot[RPW][DB];
+    float m_run[RPW], l_run[RPW];
     #pragma unroll
-    for (int d = 0; d < DB; d++) ot[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = a.sink ? a.sink[h] : WM_NEG_BIG, l_run = a.sink ? 1.0f : 0.0f;
+    for (int n = 0; n < RPW; n++)
+    {
+        #pragma unroll
+        for (int d = 0; d < DB; d++) ot[n][d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        m_run[n] = a.sink ? a.sink[h] : WM_NEG_BIG; l_run[n] = a.sink ? 1.0f : 0.0f;
+    }
 
     long long krow[KPT], vrow[VPT];                             // rows of the NEXT step's pieces
     u32x4 kreg[KPT], vreg[VPT];
@@ -508,112 +517,130 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
             }
             if (!wave_live || !any) continue;
         }
-        f32x4 st[NBLK];
+        f32x4 st[RPW][NBLK];
         #pragma unroll
         for (int blk = 0; blk < NBLK; blk++)
         {
-            st[blk] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int n = 0; n < RPW; n++) st[n][blk] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
             const u16* kf = k_lds + (16 * blk + qi) * KSTR + 8 * g;
             #pragma unroll
-            for (int kk = 0; kk < KK; kk++) st[blk] = mfma_16x16x32_bf16(*(const u32x4*)(kf + 32 * kk), qb[kk], st[blk]);
-        }
-        float sc[4 * NBLK];
-        float m_loc = WM_NEG_BIG;
-        #pragma unroll
-        for (int blk = 0; blk < NBLK; blk++)
-            #pragma unroll
-            for (int r = 0; r < 4; r++)
+            for (int kk = 0; kk < KK; kk++)
             {
-                const int e = k0 + 16 * blk + 4 * g + r;
-                const int j = j_lo + (e - NB);
-                const bool valid = e < total && (e < NB ? e < my_nb : (j <= qpos && j >= my_lo));
-                const float v = valid ? st[blk][r] : WM_NEG_BIG;
-                sc[blk * 4 + r] = v;
-                m_loc = fmaxf(m_loc, v);
+                const u32x4 kv = *(const u32x4*)(kf + 32 * kk);
+                #pragma unroll
+                for (int n = 0; n < RPW; n++) st[n][blk] = mfma_16x16x32_bf16(kv, qb[n][kk], st[n][blk]);
             }
-        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 16));
-        m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 32));
-        const float m_new = fmaxf(m_run, m_loc);
-        const float alpha = expf(m_run - m_new);
-        float p_sum = 0.0f;
-        u32x4 pb[NBLK / 2];
-        #pragma unroll
-        for (int e2 = 0; e2 < 2 * NBLK; e2++)
-        {
-            const float pa = sc[2 * e2] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2] - m_new) : 0.0f;
-            const float pc = sc[2 * e2 + 1] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2 + 1] - m_new) : 0.0f;
-            p_sum += pa + pc;
-            pb[e2 / 4][e2 % 4] = wm_pack2(pa, pc);
         }
-        p_sum += shfl_xor_f32(p_sum, 16);
-        p_sum += shfl_xor_f32(p_sum, 32);
-        l_run = l_run * alpha + p_sum;
-        m_run = m_new;
+        u32x4 pb[RPW][NBLK / 2];
+        float alpha[RPW];
+        #pragma unroll
+        for (int n = 0; n < RPW; n++)
+        {
+            float sc[4 * NBLK];
+            float m_loc = WM_NEG_BIG;
+            #pragma unroll
+            for (int blk = 0; blk < NBLK; blk++)
+                #pragma unroll
+                for (int r = 0; r < 4; r++)
+                {
+                    const int e = k0 + 16 * blk + 4 * g + r;
+                    const int j = j_lo + (e - NB);
+                    const bool valid = e < total && (e < NB ? e < my_nb[n] : (j <= qpos[n] && j >= my_lo[n]));
+                    const float v = valid ? st[n][blk][r] : WM_NEG_BIG;
+                    sc[blk * 4 + r] = v;
+                    m_loc = fmaxf(m_loc, v);
+                }
+            m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 16));
+            m_loc = fmaxf(m_loc, shfl_xor_f32(m_loc, 32));
+            const float m_new = fmaxf(m_run[n], m_loc);
+            alpha[n] = expf(m_run[n] - m_new);
+            float p_sum = 0.0f;
+            #pragma unroll
+            for (int e2 = 0; e2 < 2 * NBLK; e2++)
+            {
+                const float pa = sc[2 * e2] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2] - m_new) : 0.0f;
+                const float pc = sc[2 * e2 + 1] > 0.5f * WM_NEG_BIG ? expf(sc[2 * e2 + 1] - m_new) : 0.0f;
+                p_sum += pa + pc;
+                pb[n][e2 / 4][e2 % 4] = wm_pack2(pa, pc);
+            }
+            p_sum += shfl_xor_f32(p_sum, 16);
+            p_sum += shfl_xor_f32(p_sum, 32);
+            l_run[n] = l_run[n] * alpha[n] + p_sum;
+            m_run[n] = m_new;
+        }
         // O^T = alpha O^T + V^T P^T: this lane points at value row 4 g + qi / 4, features 16 d + 4 (qi % 4) .. + 3
         const u16* vbase = v_lds + (4 * g + (qi >> 2)) * VSTR + 4 * (qi & 3);
         #pragma unroll
         for (int d = 0; d < DB; d++)
         {
-            ot[d][0] *= alpha; ot[d][1] *= alpha; ot[d][2] *= alpha; ot[d][3] *= alpha;
+            #pragma unroll
+            for (int n = 0; n < RPW; n++) { ot[n][d][0] *= alpha[n]; ot[n][d][1] *= alpha[n]; ot[n][d][2] *= alpha[n]; ot[n][d][3] *= alpha[n]; }
             #pragma unroll
             for (int m2 = 0; m2 < NBLK / 2; m2++)
             {
                 const f16x4 lo = lds_read_tr16_b64((const f16*)(vbase + (32 * m2) * VSTR + 16 * d));
                 const f16x4 hi = lds_read_tr16_b64((const f16*)(vbase + (32 * m2 + 16) * VSTR + 16 * d));
                 const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-                ot[d] = mfma_16x16x32_bf16((u32x4){l2[0], l2[1], h2[0], h2[1]}, pb[m2], ot[d]);
+                const u32x4 va = {l2[0], l2[1], h2[0], h2[1]};
+                #pragma unroll
+                for (int n = 0; n < RPW; n++) ot[n][d] = mfma_16x16x32_bf16(va, pb[n][m2], ot[n][d]);
             }
         }
     }
 
     // O^T[feature 16 d + 4 g + r][query qi] / l, turned back by the row's position, gated -> out[row][head][feature]
-    if (my_row >= n_rows) return;
-    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
     #pragma unroll
-    for (int d = 0; d < DB; d++) { ot[d][0] *= inv; ot[d][1] *= inv; ot[d][2] *= inv; ot[d][3] *= inv; }
-    if (a.v_rot)
+    for (int n = 0; n < RPW; n++)
     {
-        const float fpos = (float)qpos;
-        if (a.interleaved)
+        if (my_row[n] >= n_rows) continue;
+        const float inv = l_run[n] > 0.0f ? 1.0f / l_run[n] : 0.0f;
+        #pragma unroll
+        for (int d = 0; d < DB; d++) { ot[n][d][0] *= inv; ot[n][d][1] *= inv; ot[n][d][2] *= inv; ot[n][d][3] *= inv; }
+        if (a.v_rot)
         {
-            #pragma unroll
-            for (int d = 0; d < DB; d++)
+            const float fpos = (float)qpos[n];
+            if (a.interleaved)
+            {
                 #pragma unroll
-                for (int r = 0; r < 4; r += 2)
-                {
-                    const float ang = fpos * a.vfreq[(16 * d + 4 * g + r) / 2];
-                    const float c = cosf(ang), sn = sinf(ang);
-                    const float u = ot[d][r], v = ot[d][r + 1];
-                    ot[d][r] = u * c + v * sn; ot[d][r + 1] = v * c - u * sn;
-                }
-        }
-        else
-        {
-            #pragma unroll
-            for (int d = 0; d < DB / 2; d++)
+                for (int d = 0; d < DB; d++)
+                    #pragma unroll
+                    for (int r = 0; r < 4; r += 2)
+                    {
+                        const float ang = fpos * a.vfreq[(16 * d + 4 * g + r) / 2];
+                        const float c = cosf(ang), sn = sinf(ang);
+                        const float u = ot[n][d][r], v = ot[n][d][r + 1];
+                        ot[n][d][r] = u * c + v * sn; ot[n][d][r + 1] = v * c - u * sn;
+                    }
+            }
+            else
+            {
                 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                {
-                    const float ang = fpos * a.vfreq[16 * d + 4 * g + r];
-                    const float c = cosf(ang), sn = sinf(ang);
-                    const float u = ot[d][r], v = ot[d + DB / 2][r];
-                    ot[d][r] = u * c + v * sn; ot[d + DB / 2][r] = v * c - u * sn;
-                }
+                for (int d = 0; d < DB / 2; d++)
+                    #pragma unroll
+                    for (int r = 0; r < 4; r++)
+                    {
+                        const float ang = fpos * a.vfreq[16 * d + 4 * g + r];
+                        const float c = cosf(ang), sn = sinf(ang);
+                        const float u = ot[n][d][r], v = ot[n][d + DB / 2][r];
+                        ot[n][d][r] = u * c + v * sn; ot[n][d + DB / 2][r] = v * c - u * sn;
+                    }
+            }
         }
-    }
-    u16* op = (u16*)a.out + ((long long)qrow * a.H + h) * VDIM + 4 * g;
-    const float* gt = a.gate ? a.gate + (long long)qrow * a.ldg + h * VDIM + 4 * g : nullptr;
-    #pragma unroll
-    for (int d = 0; d < DB; d++)
-    {
-        f32x4 y = ot[d];
-        if (gt)
+        u16* op = (u16*)a.out + ((long long)qrow[n] * a.H + h) * VDIM + 4 * g;
+        const float* gt = a.gate ? a.gate + (long long)qrow[n] * a.ldg + h * VDIM + 4 * g : nullptr;
+        #pragma unroll
+        for (int d = 0; d < DB; d++)
         {
-            const f32x4 gv = *(const f32x4*)(gt + 16 * d);
-            #pragma unroll
-            for (int r = 0; r < 4; r++) y[r] *= 1.0f / (1.0f + expf(-gv[r]));
+            f32x4 y = ot[n][d];
+            if (gt)
+            {
+                const f32x4 gv = *(const f32x4*)(gt + 16 * d);
+                #pragma unroll
+                for (int r = 0; r < 4; r++) y[r] *= 1.0f / (1.0f + expf(-gv[r]));
+            }
+            *(u32x2*)(op + 16 * d) = (u32x2){wm_pack2(y[0], y[1]), wm_pack2(y[2], y[3])};
         }
-        *(u32x2*)(op + 16 * d) = (u32x2){wm_pack2(y[0], y[1]), wm_pack2(y[2], y[3])};
     }
 }
 
@@ -622,11 +649,13 @@ static int wa_log2_exact(int x) { int sh = 0; while ((1 << sh) < x) sh++; return
 template <int DIM, int VDIM>
 static void wm_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
 {
+    // RPW = 1.  (RPW = 2 -- tiles of 128 positions, every LDS fragment feeding two products -- was built and measured slower at
+    // head size 128: 217 against 107 us at 2048 rows x 16 heads; its 233 registers left arrays in scratch memory.)
     static bool attr_done[EXL2_MAX_DEVICES];
     const size_t lds = ((size_t)WM_BK * (DIM + 8) + (size_t)WM_BK * (VDIM + 16)) * 2;
     if (exl2_first_on_device(attr_done))
-        (void)hipFuncSetAttribute((const void*)window_attn_mfma_kernel<DIM, VDIM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    LAUNCH((window_attn_mfma_kernel<DIM, VDIM>), dim3(tiles, m.w.H), dim3(256), lds, s, m);
+        (void)hipFuncSetAttribute((const void*)window_attn_mfma_kernel<DIM, VDIM, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    LAUNCH((window_attn_mfma_kernel<DIM, VDIM, 1>), dim3(tiles, m.w.H), dim3(256), lds, s, m);
 }
 
 // Decoded tokens: workgroup = one row x one key / value head.  The 16 query columns of the products are the query heads that

@@ -14,6 +14,8 @@ import torch
 from .cache import PAGE_SIZE, PagePool
 from .layered import SPAN_CHUNK, StepBatch
 
+PROMPT_TILE = 64                                          # rows per tile of a prompt portion (csrc/window_attn.hip: 16 query rows per wave)
+
 
 class Engine:
     def __init__(self, model, max_tokens: int, max_seqs: int = 4, page_size: int = PAGE_SIZE, graphs: bool | None = None):
@@ -41,7 +43,7 @@ class Engine:
         back after the step.  Returns fp32 logits [n wanted, vocab] on the device, or None."""
         ids, seq, pos, want_rows = [], [], [], []
         t16_row0, t16_rows, t1_row0, t1_maxpos = [], [], [], 0
-        t64_row0, t64_rows = [], []
+        prompt_spans = []
         spans = []
         seen = set()
         for rid, tokens, want in entries:
@@ -57,9 +59,8 @@ class Engine:
             start = self.pool.extend(slot, n)
             base = len(ids)
             spans.append((base, n, slot, start))
-            for i in range(0, n if n > 1 else 0, 64):
-                t64_row0.append(base + i)
-                t64_rows.append(min(64, n - i))
+            if n > 1:
+                prompt_spans.append((base, n))
             if n == 1:
                 t1_row0.append(base)
                 t1_maxpos = max(t1_maxpos, start)
@@ -89,9 +90,13 @@ class Engine:
             sp = torch.tensor([[s[0] for s in spans], [s[1] for s in spans], chunk0], dtype=torch.int32).to(dev)
             batch.spans_dev = (sp[0], sp[1], len(spans), max(s[1] for s in spans))
             batch.span_chunks = (sp[2], SPAN_CHUNK, total)
-            if t64_row0:
-                t64 = torch.tensor([t64_row0, t64_rows], dtype=torch.int32).to(dev)
-                batch.tiles64 = (t64[0], t64[1], len(t64_row0))
+            if prompt_spans:
+                # tiles of consecutive positions for the tiled attention kernels
+                size = PROMPT_TILE
+                row0 = [b + i for b, n in prompt_spans for i in range(0, n, size)]
+                nrow = [min(size, n - i) for b, n in prompt_spans for i in range(0, n, size)]
+                tl = torch.tensor([row0, nrow], dtype=torch.int32).to(dev)
+                batch.prompt_tiles = (tl[0], tl[1], len(row0), size)
             if t16_row0:
                 t16 = torch.tensor([t16_row0, t16_rows], dtype=torch.int32).to(dev)
                 batch.tiles16 = (t16[0], t16[1], len(t16_row0))

@@ -85,8 +85,8 @@ class StepBatch:
     # (row0 int32 [n], rows int32 [n], n) and single decoded tokens (row0 int32 [n], n, largest position among them)
     tiles16: tuple | None = None
     tiles1: tuple | None = None
-    # the portions of prompts again in tiles of <= 64 consecutive positions (row0 int32 [n], rows int32 [n], n)
-    tiles64: tuple | None = None
+    # the portions of prompts again in tiles of <= 64 consecutive positions (row0 int32 [n], rows int32 [n], n, tile size)
+    prompt_tiles: tuple | None = None
     # the runs of consecutive rows that one sequence brings (recurrent mixers walk them in order): (first row int32 [n],
     # rows int32 [n], n, longest run)
     spans_dev: tuple | None = None

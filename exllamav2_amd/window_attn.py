@@ -101,11 +101,12 @@ class WindowAttention:
         o = m.buf("attn.o", (rows, H * vd), m.dtype)
         common = (q, st.k, st.v, st.k_pool, st.v_pool, self.sink, f, ncat, self.off_g, self.vfreq, self.rotate_values, self.interleaved,
                   batch.row_seq, batch.row_pos, batch.block_table, page, self.pool, o)
-        if self.tiles_ok and (batch.tiles64 is not None or batch.tiles1 is not None):
-            # matrix-core kernels: portions of prompts as tiles of <= 64 positions x one head per workgroup, decoded tokens as one row x
-            # one key / value head per workgroup (its query heads share the pass over the keys)
-            if batch.tiles64 is not None:
-                ext.window_attn_tiles(*common, batch.tiles64, 64, H, G, dim, vd, self.window)
+        if self.tiles_ok and (batch.prompt_tiles is not None or batch.tiles1 is not None):
+            # matrix-core kernels: portions of prompts as tiles of <= 64 positions x one head per workgroup, decoded tokens as one
+            # row x one key / value head per workgroup (its query heads share the pass over the keys)
+            if batch.prompt_tiles is not None:
+                row0, nrow, n, size = batch.prompt_tiles
+                ext.window_attn_tiles(*common, (row0, nrow, n), size, H, G, dim, vd, self.window)
             if batch.tiles1 is not None:
                 row0, n, max_pos = batch.tiles1
                 # the longest key list among the rows: window tokens + pooled blocks; its steps of 128 entries go to up to 16 workgroups

@@ -97,7 +97,7 @@ def test_causal_conv_over_spans_and_steps(be, taps):
     w, b = OH.bf16_round(rng.standard_normal((C, taps))), OH.bf16_round(rng.standard_normal(C))
     tail = torch.full((3, max(taps - 1, 1), C), 7.0, dtype=F32, device=be.device)          # stale values of an earlier user
     hist = {1: np.zeros((0, C)), 2: np.zeros((0, C))}
-    for step in ([(1, 2), (2, 1)], [(2, 40), (1, 1)], [(1, 1)], [(1, 5), (2, 3)], [(2, 1)]):
+    for step in ([(1, 2), (2, 1)], [(2, 40), (1, 1)], [(1, 1)], [(1, 5), (2, 3)], [(2, 1)], [(1, 70), (2, 2)], [(2, 3)]):
         lens = [n for _s, n in step]
         rows = sum(lens)
         f = rng.standard_normal((rows, ld)).astype(np.float32)
@@ -262,8 +262,9 @@ class KernelAttention:
                 be.ext.window_attn_tiles(*common, (ints(be, [0]), None, 1), 1, H, G, dim, vd, m["mask"]["size"], nsplit=nsplit,
                                          part_o=part_o, part_ml=part_ml)
             else:
-                row0 = list(range(0, rows, 64))
-                be.ext.window_attn_tiles(*common, (ints(be, row0), ints(be, [min(64, rows - r) for r in row0]), len(row0)), 64, H, G, dim, vd,
+                size = 64
+                row0 = list(range(0, rows, size))
+                be.ext.window_attn_tiles(*common, (ints(be, row0), ints(be, [min(size, rows - r) for r in row0]), len(row0)), size, H, G, dim, vd,
                                          m["mask"]["size"])
         else:
             be.ext.window_attn(*common, rows, H, G, dim, vd, m["mask"]["size"])
@@ -331,7 +332,7 @@ def test_matrix_core_attention_against_the_oracle(be, shape):
     page = shape.pop("page")
     m = OH.attn_mixer(**shape)["mixer"]
     rng = np.random.default_rng(shape["dim"] + shape["size"])
-    T, H, G, dim, vd = 230, m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    T, H, G, dim, vd = 370, m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     rnd = lambda *s: OH.bf16_round(rng.standard_normal(s))
     q, k, v, gate = rnd(T, H, dim), rnd(T, G, dim), rnd(T, G, vd), rnd(T, H, vd)
     q_scale = (m["scale"] * (1 + 0.3 * rng.standard_normal(H))).astype(np.float32)
@@ -342,7 +343,7 @@ def test_matrix_core_attention_against_the_oracle(be, shape):
     table[1, :] = rng.permutation(pages)
     ka = KernelAttention(be, BF16, m, page, pages, table)
     got, at = [], 0
-    for n in [1, 1, 30, 1, 100, 17, 1, 63, 1, 14, 1]:
+    for n in [1, 1, 30, 1, 100, 17, 1, 63, 1, 14, 1, 140]:
         sl = slice(at, at + n)
         got.append(ka.step(q[sl], k[sl], v[sl], gate[sl], [1] * n, list(range(at, at + n)), q_scale, sink, tiles=True))
         at += n
