@@ -324,7 +324,10 @@ def test_attention_kernels_against_the_oracle(be, dtype, shape):
                                    dict(heads=3, kv_heads=3, dim=128, vdim=64, size=33, pool=5, dims=32, page=7),
                                    dict(heads=2, kv_heads=2, dim=96, vdim=96, size=200, pool=64, dims=32, page=256),
                                    dict(heads=2, kv_heads=1, dim=64, vdim=128, size=1, pool=1, dims=2, page=3),
-                                   dict(heads=34, kv_heads=2, dim=32, vdim=32, size=20, pool=6, dims=8, page=32)])
+                                   dict(heads=34, kv_heads=2, dim=32, vdim=32, size=20, pool=6, dims=8, page=32),
+                                   dict(heads=2, kv_heads=1, dim=128, vdim=128, size=50, pool=8, dims=64, page=32),
+                                   dict(heads=2, kv_heads=2, dim=192, vdim=128, size=90, pool=32, dims=96, page=128, scaling=None),
+                                   dict(heads=1, kv_heads=1, dim=256, vdim=256, size=30, pool=4, dims=32, page=16)])
 def test_matrix_core_attention_against_the_oracle(be, shape):
     """the bfloat16 tile kernel over 230 positions fed in steps of 1 .. 100 rows (tiles that start inside windows, blocks and pages,
     single decoded rows, a step of more than one tile): every position's output equals the float64 form"""
