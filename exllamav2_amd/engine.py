@@ -123,6 +123,10 @@ class Engine:
             st["batch"] = StepBatch(st["inputs"][0], st["inputs"][1], st["inputs"][2], self.pool.device_table(), ar, b, b,
                                     tiles1=(ar, b, cap - 1), spans_dev=(ar, torch.ones_like(ar), b, 1))
             self._decode[b] = st
+        if st["graph"] is not None and st.get("epoch") != getattr(m, "scratch_epoch", 0):
+            # a larger step has moved a scratch buffer since the capture: the graph holds the old addresses
+            ext.graph_free(st["graph"])
+            st["graph"], st["runs"] = None, 1
         host = torch.tensor([ids, seq, pos], dtype=torch.int32)
         if self._stream is None:                                   # (no GPU: the same batch, eagerly)
             st["inputs"].copy_(host)
@@ -144,6 +148,7 @@ class Engine:
                         st["logits"] = m.step(st["batch"], self.cache)    # recorded, not run
                     finally:
                         st["graph"] = ext.graph_end_capture(self._stream.cuda_stream)
+                        st["epoch"] = getattr(m, "scratch_epoch", 0)
                         m.frozen = False
             else:
                 ext.graph_launch(st["graph"], self._stream.cuda_stream)

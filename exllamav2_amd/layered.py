@@ -107,6 +107,7 @@ class LayeredModel:
         self.layers = []
         self.loaded = False
         self._scratch = {}
+        self.scratch_epoch = 0                            # counts (re)allocations of scratch buffers: a graph captured before one is stale
         self.frozen = False                               # True while a step is being captured into a graph: scratch may not grow
 
     def buf(self, tag: str, shape, dtype) -> torch.Tensor:
@@ -122,6 +123,7 @@ class LayeredModel:
                 raise RuntimeError(f"scratch buffer '{tag}' would have to grow while a step is being captured")
             t = torch.empty((max(n, 1),), dtype=dtype, device=self.device)
             self._scratch[tag] = t
+            self.scratch_epoch += 1
         return t[:n].view(*shape)
 
     # ---- loading --------------------------------------------------------------------------------------------------------------

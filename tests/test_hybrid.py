@@ -541,6 +541,37 @@ def test_decode_steps_as_graphs(be, dtype):
     eng.close()
 
 
+def test_decode_graphs_survive_a_larger_step(be):
+    """decode-only steps are captured while the scratch buffers are still small; a longer portion then moves the buffers; the decode
+    steps after it must not replay the old addresses"""
+    cfg = CONFIGS["wide"]()
+    W = OH.random_model(cfg, seed=41)
+    rng = np.random.default_rng(42)
+    reqs = {r: list(map(int, rng.integers(0, cfg["vocab"], size=n))) for r, n in (("a", 12), ("b", 90), ("c", 10))}
+    oracle = OH.Oracle(cfg, W)
+    want = {r: oracle.feed(r, t) for r, t in reqs.items()}
+    eng = make_engine(be, cfg, W, BF16, max_tokens=160, page=16, graphs=True)
+    got = {r: {} for r in reqs}
+
+    def step(parts, end=()):
+        lg = be.n(eng.step([(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in parts], end))
+        k = 0
+        for r, lo, hi in parts:
+            for p in range(lo, hi):
+                got[r][p] = lg[k]; k += 1
+
+    for i in range(5):
+        step([("a", i, i + 1)])                                  # one token per step from the first token on: captured at the third
+    step([("b", 0, 80), ("a", 5, 6)])                            # 81 rows: every scratch buffer grows
+    for i in range(6, 12):
+        step([("a", i, i + 1)])
+    for i in range(80, 90):
+        step([("b", i, i + 1), ("c", i - 80, i - 79)])
+    for r in reqs:
+        assert rel_err(np.stack([got[r][p] for p in range(len(reqs[r]))]), want[r]) <= TOL[BF16], r
+    eng.close()
+
+
 def crafted_model(window, pool, seed=31):
     """one attention layer between a state-space layer and a feed-forward, made so that token 0's query matches token 1's key and
     nothing else: queries read inputs 0-3, keys inputs 4-7 through the same matrix, values the other inputs; token 0 is marked in
