@@ -35,6 +35,7 @@ struct ConvArgs
     float* tail;                             // [slots, taps - 1, channels]: inputs of the last taps - 1 positions of every sequence
     const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
     int channels, taps;
+    int roll_tail;                           // every span is one walk: the convolution kernel rolls the tails itself
 };
 
 // grid (channel blocks, token chunks, spans): thread = one channel over CONV_TOKENS consecutive rows of a span; the window of the
@@ -88,9 +89,31 @@ KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
         }
         a.out[(long long)(r0 + t0 + i) * a.ldo + c] = ss_silu(acc);
     }
+    if (a.roll_tail && a.taps > 1)
+    {
+        // the span is this one walk, so this thread alone reads and writes channel c of the slot's tail: the inputs of the
+        // sequence's last taps - 1 positions (rows of the span where it is long enough, the old tail shifted where it is not)
+        float* tl = a.tail + (long long)a.row_seq[r0] * (a.taps - 1) * a.channels;
+        float nv[MAXT];
+        #pragma unroll
+        for (int k = 0; k < MAXT - 1; k++)
+        {
+            nv[k] = 0.0f;
+            if (k < a.taps - 1)
+            {
+                const int tok = n - (a.taps - 1) + k;
+                if (tok >= 0) nv[k] = a.in[(long long)(r0 + tok) * a.ld + c];
+                else if (pos0 + tok >= 0) nv[k] = tl[(long long)(a.taps - 1 + tok) * a.channels + c];
+            }
+        }
+        #pragma unroll
+        for (int k = 0; k < MAXT - 1; k++)
+            if (k < a.taps - 1) tl[(long long)k * a.channels + c] = nv[k];
+    }
 }
 
-// The tails after the step: for every span the inputs of its last taps - 1 positions (rows of the span where it is long enough,
+// The tails after a step with spans of several walks (the first walk reads the old tail while the last would write the new one, so
+// the roll is a launch of its own there): for every span the inputs of its last taps - 1 positions (rows of the span where it is long enough,
 // the old tail shifted where it is not).  One thread per (span, channel) reads all it needs before it writes.
 KERNEL void __launch_bounds__(256) conv_tail_kernel(const ConvArgs a)
 {
@@ -552,6 +575,7 @@ extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const
     ConvArgs a;
     a.in = in; a.ld = ld; a.w = w; a.bias = bias; a.out = out; a.ldo = ldo; a.tail = tail; a.span_row0 = span_row0; a.span_rows = span_rows;
     a.row_seq = row_seq; a.row_pos = row_pos; a.channels = channels; a.taps = taps;
+    a.roll_tail = max_span_rows <= CONV_TOKENS;
     const dim3 grid((channels + 255) / 256, (max_span_rows + CONV_TOKENS - 1) / CONV_TOKENS, spans);
     if (dtype == 0)
     {
@@ -565,7 +589,7 @@ extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const
         else if (taps <= 8) LAUNCH((conv_silu_kernel<float, 8>), grid, dim3(256), 0, stream, a);
         else LAUNCH((conv_silu_kernel<float, CONV_MAX_TAPS>), grid, dim3(256), 0, stream, a);
     }
-    if (taps > 1) LAUNCH(conv_tail_kernel, dim3((channels + 255) / 256, spans), dim3(256), 0, stream, a);
+    if (taps > 1 && !a.roll_tail) LAUNCH(conv_tail_kernel, dim3((channels + 255) / 256, spans), dim3(256), 0, stream, a);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }
